@@ -10,9 +10,14 @@ import pytest
 ROOT = Path(__file__).resolve().parent.parent
 
 
-def declared_symbols():
+HYBRID_HEADER = "tinyllm_hybrid.h"  # the layer-list engine: a library and a binding of its own
+
+
+def declared_symbols(hybrid: bool = False):
     names = set()
     for header in (ROOT / "include").glob("*.h"):
+        if (header.name == HYBRID_HEADER) != hybrid:
+            continue
         text = re.sub(r"/\*.*?\*/", "", header.read_text(), flags=re.S)
         names.update(re.findall(r"\b(tl_[a-z0-9_]+)\s*\(", text))
     return sorted(names)
@@ -30,6 +35,19 @@ def test_every_declared_symbol_is_exported_and_bound(built_libs):
         assert name in ext._SIGNATURES, f"{name} has no ctypes signature in tiny_llm_ext_hip"
     for name in ext._SIGNATURES:
         assert name in declared, f"{name} is bound in Python but not declared in include/*.h"
+
+
+def test_layer_list_engine_symbols_are_exported_and_bound(built_libs):
+    import tiny_llm_ext_hybrid as hyb
+
+    lib = ctypes.CDLL(hyb.library_path())
+    declared = declared_symbols(hybrid=True)
+    assert len(declared) >= 15
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/{HYBRID_HEADER} but not exported by libtinyllm_hybrid.so"
+        assert name in hyb.SIGNATURES, f"{name} has no ctypes signature in tiny_llm_ext_hybrid"
+    for name in hyb.SIGNATURES:
+        assert name in declared, f"{name} is bound in Python but not declared in include/{HYBRID_HEADER}"
 
 
 def test_reference_operator_surface(built_libs):

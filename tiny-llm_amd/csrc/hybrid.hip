@@ -1,0 +1,693 @@
+// The layer-list engine (include/tinyllm_hybrid.h): host side.
+//   * layer runs: the layer list unrolled over the loop passes; every run owns its K/V pages (attention) or state slots (delta)
+//   * page pool + slots (page_pool.h), block table mirrored to the device when it changes
+//   * one packed step function for prefill chunks, decode tokens and mixtures; a device-resident greedy decode loop on top of it,
+//     captured in a hipGraph per slot list
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/tinyllm_hybrid.h"
+#include "common.h"
+#include "hybrid_kernels.h"
+#include "page_pool.h"
+
+#define HY_HIP(call)                                                                                   \
+    do {                                                                                               \
+        hipError_t e__ = (call);                                                                       \
+        if (e__ != hipSuccess) return ::tl::fail(TL_ERR_HIP, std::string(#call) + ": " + hipGetErrorString(e__)); \
+    } while (0)
+#define HY_TRY(call)              \
+    do {                          \
+        int s__ = (call);         \
+        if (s__ != 0) return s__; \
+    } while (0)
+
+namespace tl {
+namespace hy {
+
+struct Run {
+    int layer = 0;
+    int pass = -1;            // loop pass this run belongs to, -1 outside the loop
+    bool enters_pass = false; // the loop-entry projection + pass offset come right before this run
+    void *kpool = nullptr, *vpool = nullptr;      // attention: [pages, G, page, dim] / [pages, G, page, vdim] of the engine dtype
+    float *state = nullptr, *conv_state = nullptr; // delta: [slots, H, dim, vdim] / [slots, taps-1, C]
+};
+
+struct Meta {  // device int32 arrays of one step
+    int32_t *tokens, *row_seq, *row_pos, *seq_row0, *seq_slot, *want_rows, *want_slot;
+};
+
+}  // namespace hy
+}  // namespace tl
+
+struct tl_hybrid {
+    tl_hybrid_config cfg{};
+    std::vector<tl_hybrid_layer> layers;
+    std::vector<tl::hy::Run> runs;
+    std::vector<float *> inv_freq;  // per layer (attention with rotary positions), device
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    int device = 0;
+    std::unique_ptr<tl::PagePool> pool;
+    bool table_dirty = true;
+    int32_t *table_dev = nullptr;
+    // workspace
+    float *x = nullptr, *x0 = nullptr, *proj = nullptr, *qbuf = nullptr, *conv_out = nullptr, *obuf = nullptr, *logits = nullptr;
+    void *h = nullptr, *cat = nullptr, *cat2 = nullptr, *hsel = nullptr;
+    int ld_proj = 0, ld_cat = 0;
+    int32_t *meta_dev = nullptr, *meta_host = nullptr;  // step metadata (host side pinned)
+    int32_t *dmeta_dev = nullptr;                        // decode-loop metadata (its own copy: captured graphs point into it)
+    int32_t *ctx_dev = nullptr, *pending_dev = nullptr, *argmax_dev = nullptr;
+    tl::hy::Meta meta{}, dmeta{};
+    std::vector<int32_t> pending_host_valid;
+    int last_rows = 0;
+    // trace of the residual stream
+    bool trace = false;
+    float *trace_buf = nullptr;
+    int trace_rows = 0;
+    // decode graphs by slot list
+    std::map<std::vector<int>, hipGraphExec_t> graphs;
+    std::vector<int> dmeta_slots;  // the slot list dmeta currently describes
+    tl_hybrid_stats stats{};
+    std::vector<void *> allocs;
+};
+
+namespace tl {
+namespace hy {
+
+static size_t esize(int dtype) { return dtype == TL_HY_BF16 ? 2 : 4; }
+
+static int in_cols(const tl_hybrid_layer &L) {  // rows of w_in
+    if (L.kind == TL_MIX_ATTENTION) return L.heads * L.dim + L.kv_heads * L.dim + L.kv_heads * L.vdim + (L.gated ? L.heads * L.vdim : 0) + L.ff;
+    return 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim + 2 * L.heads + L.ff;
+}
+static int conv_channels(const tl_hybrid_layer &L) { return 2 * L.kv_heads * L.dim + L.heads * L.vdim; }
+
+template <typename T>
+static int dev_alloc(tl_hybrid *e, T **p, size_t count, bool zero = false) {
+    void *q = nullptr;
+    HY_HIP(hipMalloc(&q, std::max<size_t>(count, 1) * sizeof(T)));
+    e->allocs.push_back(q);
+    *p = (T *)q;
+    if (zero) HY_HIP(hipMemset(q, 0, std::max<size_t>(count, 1) * sizeof(T)));  // at creation only, never inside a captured region
+    return TL_OK;
+}
+
+static Meta carve(int32_t *base, int R, int S) {
+    Meta m;
+    m.tokens = base;
+    m.row_seq = base + R;
+    m.row_pos = base + 2 * R;
+    m.want_rows = base + 3 * R;
+    m.want_slot = base + 4 * R;
+    m.seq_row0 = base + 5 * R;
+    m.seq_slot = base + 5 * R + S + 1;
+    return m;
+}
+static size_t meta_ints(int R, int S) { return (size_t)5 * R + 2 * S + 2; }
+
+// out (+)= A . W^T by shape: a few rows stream the weights once per column (row kernel), more go through the MFMA tile kernel
+template <typename D>
+static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, int M, int N, int K, int epi, float alpha, const float *bias,
+                    int force, hipStream_t st) {
+    using S = typename D::storage;
+    if (M <= 0 || N <= 0) return TL_OK;
+    const int vec_ok = (K % 8 == 0) && (lda % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+    const bool rows = force == 1 || (force == 0 && M <= 8);
+    TL_REQUIRE(!rows || M <= 8, "hybrid linear: the row kernel takes at most 8 rows");
+    if (rows) {
+        dim3 grid((N + 3) / 4), block(256);
+        if (epi == 0) hipLaunchKernelGGL((gemm_rows_kernel<D, 0>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+        else if (epi == 1) hipLaunchKernelGGL((gemm_rows_kernel<D, 1>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+        else hipLaunchKernelGGL((gemm_rows_kernel<D, 2>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+    } else {
+        dim3 grid(((M + 63) / 64) * ((N + 63) / 64)), block(256);
+        if (epi == 0) hipLaunchKernelGGL((gemm_tile_kernel<D, 0>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+        else if (epi == 1) hipLaunchKernelGGL((gemm_tile_kernel<D, 1>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+        else hipLaunchKernelGGL((gemm_tile_kernel<D, 2>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+    }
+    TL_CHECK_LAUNCH("hybrid linear");
+    return TL_OK;
+}
+
+static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs) {
+    // lanes per state column R and rows per lane RPT: key_dim <= RPT * R; a workgroup takes VB columns with VB * R <= 256 threads
+    int rpt = 8;
+    while (rpt < 128 && (L.dim + rpt - 1) / rpt > 16) rpt *= 2;
+    int R = 1;
+    while (R * rpt < L.dim) R *= 2;
+    TL_REQUIRE(R <= 64, "hybrid delta: key width above 8192 is not supported");
+    int VB = std::max(1, std::min(L.vdim, 256 / R));
+    const int threads = ((VB * R + 63) / 64) * 64;
+    int TB = (int)std::max<size_t>(1, std::min<size_t>(32, (48 * 1024 / 4) / (size_t)(2 * L.dim + VB + 2)));
+    const size_t lds = ((size_t)TB * (2 * L.dim + VB) + 2 * TB) * 4;
+    dim3 grid(L.heads, n_seqs, (L.vdim + VB - 1) / VB), block(threads);
+    const int C = conv_channels(L);
+    const int a0 = 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim, b0 = a0 + L.heads;
+#define HY_DELTA(RPT)                                                                                                                          \
+    hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, lds, e->stream, e->conv_out, C, e->proj, e->ld_proj, a0, b0, L.a_log_dev, L.dt_bias_dev, \
+                       L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim, R, VB, TB)
+    switch (rpt) {
+        case 8: HY_DELTA(8); break;
+        case 16: HY_DELTA(16); break;
+        case 32: HY_DELTA(32); break;
+        case 64: HY_DELTA(64); break;
+        default: HY_DELTA(128); break;
+    }
+#undef HY_DELTA
+    TL_CHECK_LAUNCH("hybrid delta");
+    return TL_OK;
+}
+
+// every layer run over `rows` packed rows described by m
+template <typename D>
+static int forward_t(tl_hybrid *e, const Meta &m, int rows, int n_seqs) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    hipStream_t st = e->stream;
+    const int W = c.width;
+    hipLaunchKernelGGL((embed_kernel<D>), dim3(rows), dim3(256), 0, st, m.tokens, (const S *)c.embed_dev, e->x0, e->x, W, c.vocab);
+    TL_CHECK_LAUNCH("hybrid embed");
+    for (size_t ri = 0; ri < e->runs.size(); ++ri) {
+        const Run &run = e->runs[ri];
+        const tl_hybrid_layer &L = e->layers[run.layer];
+        if (run.enters_pass) {  // x <- W_in [x ; x0] + step[pass]
+            hipLaunchKernelGGL((pack2_kernel<D>), dim3(rows), dim3(256), 0, st, e->x, e->x0, (S *)e->cat2, W);
+            TL_CHECK_LAUNCH("hybrid pack2");
+            HY_TRY(linear_t<D>(e->cat2, 2 * W, c.loop_in_dev, e->x, W, rows, W, 2 * W, 2, 1.f, c.loop_step_dev + (size_t)run.pass * W, 0, st));
+        }
+        hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(256), 0, st, e->x, L.norm_dev, L.norm_offset, c.norm_eps, (S *)e->h, W, (const int32_t *)nullptr);
+        TL_CHECK_LAUNCH("hybrid norm");
+        const int nin = in_cols(L), HV = L.heads * L.vdim;
+        HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, e->ld_proj, rows, nin, W, 0, 1.f, nullptr, 0, st));
+        if (L.kind == TL_MIX_ATTENTION) {
+            const int H = L.heads, G = L.kv_heads;
+            hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, e->ld_proj, m.row_seq, m.row_pos, m.seq_slot,
+                               e->table_dev, c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.qk_unit_rms, c.norm_eps, H, G, L.dim,
+                               L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
+            TL_CHECK_LAUNCH("hybrid attention prep");
+            const float *gate = L.gated ? e->proj + (size_t)(H + G) * L.dim + (size_t)G * L.vdim : nullptr;
+            hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(rows, H), dim3(64), (L.dim + 64) * sizeof(float), st, e->qbuf, (const S *)run.kpool,
+                               (const S *)run.vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, H, G, L.dim, L.vdim,
+                               L.scale, L.sink, gate, e->ld_proj, (S *)e->cat, e->ld_cat);
+            TL_CHECK_LAUNCH("hybrid attention");
+        } else {
+            const int C = conv_channels(L);
+            const size_t n = (size_t)rows * C;
+            hipLaunchKernelGGL(conv_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, e->ld_proj, L.conv_dev, L.conv_taps, C, m.row_seq,
+                               m.seq_row0, m.seq_slot, run.conv_state, e->conv_out, rows);
+            TL_CHECK_LAUNCH("hybrid conv");
+            if (L.conv_taps > 1) {
+                hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)(((size_t)n_seqs * C + 255) / 256)), dim3(256), 0, st, e->proj, e->ld_proj, L.conv_taps, C,
+                                   m.seq_row0, m.seq_slot, run.conv_state, n_seqs);
+                TL_CHECK_LAUNCH("hybrid conv state");
+            }
+            HY_TRY(launch_delta(e, L, run, m, n_seqs));
+            const float *gate = e->proj + (size_t)C;
+            hipLaunchKernelGGL((delta_out_kernel<D>), dim3(rows, L.heads), dim3(64), 0, st, e->obuf, L.out_norm_dev, c.norm_eps, gate, e->ld_proj, L.heads,
+                               L.vdim, (S *)e->cat, e->ld_cat);
+            TL_CHECK_LAUNCH("hybrid delta out");
+        }
+        if (L.ff > 0) {
+            const size_t n = (size_t)rows * L.ff;
+            hipLaunchKernelGGL((ff_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, e->ld_proj, nin - L.ff, L.ff, L.ff_act,
+                               (S *)e->cat, e->ld_cat, HV, rows);
+            TL_CHECK_LAUNCH("hybrid ff act");
+        }
+        // x += m * ([mixer out ; ff act] . [W_o | W_down]^T)
+        HY_TRY(linear_t<D>(e->cat, e->ld_cat, L.w_out_dev, e->x, W, rows, W, HV + L.ff, 1, c.residual_mult, nullptr, 0, st));
+        if (e->trace && e->trace_buf && rows <= c.max_rows)
+            HY_HIP(hipMemcpyAsync(e->trace_buf + ri * (size_t)c.max_rows * W, e->x, (size_t)rows * W * 4, hipMemcpyDeviceToDevice, st));
+    }
+    return TL_OK;
+}
+
+// final norm on the wanted rows, head product, argmax (and the slots' next input tokens)
+template <typename D>
+static int head_t(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    if (n_want <= 0) return TL_OK;
+    hipLaunchKernelGGL((norm_kernel<D>), dim3(n_want), dim3(256), 0, e->stream, e->x, c.final_norm_dev, c.final_norm_offset, c.norm_eps, (S *)e->hsel, c.width,
+                       (const int32_t *)m.want_rows);
+    TL_CHECK_LAUNCH("hybrid final norm");
+    HY_TRY(linear_t<D>(e->hsel, c.width, c.head_dev, e->logits, c.vocab, n_want, c.vocab, c.width, 0, 1.f, nullptr, 0, e->stream));
+    hipLaunchKernelGGL(argmax_kernel, dim3(n_want), dim3(256), 0, e->stream, e->logits, c.vocab, e->argmax_dev, set_pending ? m.want_slot : (const int32_t *)nullptr,
+                       e->pending_dev);
+    TL_CHECK_LAUNCH("hybrid argmax");
+    return TL_OK;
+}
+
+static int forward(tl_hybrid *e, const Meta &m, int rows, int n_seqs) {
+    return e->cfg.dtype == TL_HY_BF16 ? forward_t<BF16>(e, m, rows, n_seqs) : forward_t<F32>(e, m, rows, n_seqs);
+}
+static int head(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
+    return e->cfg.dtype == TL_HY_BF16 ? head_t<BF16>(e, m, n_want, set_pending) : head_t<F32>(e, m, n_want, set_pending);
+}
+
+static int sync_table(tl_hybrid *e) {
+    if (!e->table_dirty) return TL_OK;
+    const auto &t = e->pool->table();
+    // the pageable source is consumed before the call returns (no pinned staging to keep alive)
+    HY_HIP(hipMemcpyAsync(e->table_dev, t.data(), t.size() * 4, hipMemcpyHostToDevice, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    e->table_dirty = false;
+    return TL_OK;
+}
+
+static int check_slots(tl_hybrid *e, int n_seqs, const int *slots) {
+    TL_REQUIRE(n_seqs >= 1 && n_seqs <= e->cfg.max_slots, "hybrid: between 1 and max_slots sequences per step");
+    std::vector<char> seen(e->cfg.max_slots, 0);
+    for (int i = 0; i < n_seqs; ++i) {
+        TL_REQUIRE(slots[i] >= 0 && slots[i] < e->cfg.max_slots, "hybrid: slot out of range");
+        TL_REQUIRE(e->pool->live(slots[i]), "hybrid: slot holds no sequence");
+        TL_REQUIRE(!seen[slots[i]], "hybrid: a slot appears twice in one step");
+        seen[slots[i]] = 1;
+    }
+    return TL_OK;
+}
+
+// pages for `extra[i]` more tokens in slots[i]: all or nothing
+static int reserve_all(tl_hybrid *e, int n_seqs, const int *slots, const int *extra) {
+    long need = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        const int mi = e->pool->missing(slots[i], e->pool->context(slots[i]) + extra[i]);
+        TL_REQUIRE(mi >= 0, "hybrid: sequence exceeds max_pages_per_seq * page_size tokens");
+        need += mi;
+    }
+    TL_REQUIRE(need <= e->pool->free_pages(), "hybrid: KV page pool exhausted");
+    for (int i = 0; i < n_seqs; ++i)
+        if (e->pool->reserve(slots[i], e->pool->context(slots[i]) + extra[i])) e->table_dirty = true;
+    return TL_OK;
+}
+
+}  // namespace hy
+}  // namespace tl
+
+using namespace tl;
+using namespace tl::hy;
+
+extern "C" const char *tl_last_error(void);
+extern "C" const char *tl_hybrid_last_error(void) { return tl_last_error(); }
+
+extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_layer *layers, void *stream, tl_hybrid **out) {
+    TL_REQUIRE(cfg && layers && out, "hybrid_create: null argument");
+    const tl_hybrid_config &c = *cfg;
+    TL_REQUIRE(c.dtype == TL_HY_BF16 || c.dtype == TL_HY_F32, "hybrid_create: dtype must be bfloat16 or float32");
+    TL_REQUIRE(c.width > 0 && c.vocab > 0 && c.num_layers > 0, "hybrid_create: width, vocab and num_layers must be positive");
+    TL_REQUIRE(c.parallel_block == 1, "hybrid_create: only the parallel block (one norm, mixer + feed-forward) is implemented");
+    TL_REQUIRE(c.page_size > 0 && c.num_pages > 0 && c.max_slots > 0 && c.max_pages_per_seq > 0 && c.max_rows > 0, "hybrid_create: pool sizes must be positive");
+    TL_REQUIRE(c.embed_dev && c.final_norm_dev && c.head_dev, "hybrid_create: embed, final norm and head are required");
+    const bool looped = c.loop_times > 1 || (c.loop_times == 1 && c.loop_stop > c.loop_start);
+    if (looped) {
+        TL_REQUIRE(c.loop_start >= 0 && c.loop_stop > c.loop_start && c.loop_stop <= c.num_layers, "hybrid_create: loop range outside the layer list");
+        TL_REQUIRE(c.loop_in_dev && c.loop_step_dev, "hybrid_create: a loop needs its entry projection and pass offsets");
+    }
+    auto e = std::make_unique<tl_hybrid>();
+    e->cfg = c;
+    e->layers.assign(layers, layers + c.num_layers);
+    HY_HIP(hipGetDevice(&e->device));
+    if (stream) e->stream = (hipStream_t)stream;
+    else {
+        HY_HIP(hipDeviceSynchronize());
+        HY_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
+        e->owns_stream = true;
+    }
+    int max_in = 0, max_cat = 0, max_q = 0, max_c = 0, max_hv = 0;
+    for (int i = 0; i < c.num_layers; ++i) {
+        const tl_hybrid_layer &L = e->layers[i];
+        TL_REQUIRE(L.kind == TL_MIX_ATTENTION || L.kind == TL_MIX_DELTA, "hybrid_create: unknown mixer kind");
+        TL_REQUIRE(L.heads > 0 && L.kv_heads > 0 && L.heads % L.kv_heads == 0, "hybrid_create: heads must be a positive multiple of kv_heads");
+        TL_REQUIRE(L.dim > 0 && L.dim <= 1024 && L.vdim > 0 && L.vdim <= 256, "hybrid_create: head widths: dim 1..1024, vdim 1..256");
+        TL_REQUIRE(L.w_in_dev && L.w_out_dev && L.norm_dev && L.ff >= 0, "hybrid_create: layer matrices and norm are required");
+        if (L.kind == TL_MIX_ATTENTION) {
+            TL_REQUIRE(L.rot_dims >= 0 && L.rot_dims % 2 == 0 && L.rot_dims <= L.dim, "hybrid_create: rot_dims must be even and at most dim");
+        } else {
+            TL_REQUIRE(L.conv_taps >= 1 && L.conv_taps <= 64 && L.conv_dev && L.a_log_dev && L.dt_bias_dev && L.out_norm_dev,
+                       "hybrid_create: a delta layer needs conv taps and weights, a_log, dt_bias and its output norm");
+        }
+        max_in = std::max(max_in, in_cols(L));
+        max_cat = std::max(max_cat, L.heads * L.vdim + L.ff);
+        max_hv = std::max(max_hv, L.heads * L.vdim);
+        if (L.kind == TL_MIX_ATTENTION) max_q = std::max(max_q, L.heads * L.dim);
+        else max_c = std::max(max_c, conv_channels(L));
+    }
+    // layer runs
+    for (int i = 0; i < c.num_layers;) {
+        if (looped && i == c.loop_start) {
+            for (int t = 0; t < c.loop_times; ++t)
+                for (int j = c.loop_start; j < c.loop_stop; ++j) {
+                    Run r;
+                    r.layer = j;
+                    r.pass = t;
+                    r.enters_pass = j == c.loop_start;
+                    e->runs.push_back(r);
+                }
+            i = c.loop_stop;
+        } else {
+            Run r;
+            r.layer = i++;
+            e->runs.push_back(r);
+        }
+    }
+    tl_hybrid *p = e.get();
+    const size_t es = esize(c.dtype);
+    e->inv_freq.assign(c.num_layers, nullptr);
+    for (int i = 0; i < c.num_layers; ++i) {
+        const tl_hybrid_layer &L = e->layers[i];
+        if (L.kind != TL_MIX_ATTENTION) continue;
+        const int half = std::max(1, L.rot_dims / 2);
+        std::vector<float> f(half, 0.f);
+        for (int k = 0; k < L.rot_dims / 2; ++k) f[k] = (float)std::pow((double)L.rot_base, -2.0 * k / (double)L.rot_dims);
+        HY_TRY(dev_alloc(p, &e->inv_freq[i], half));
+        HY_HIP(hipMemcpy(e->inv_freq[i], f.data(), half * 4, hipMemcpyHostToDevice));
+    }
+    for (Run &r : e->runs) {
+        const tl_hybrid_layer &L = e->layers[r.layer];
+        if (L.kind == TL_MIX_ATTENTION) {
+            const size_t kb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.dim * es, vb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.vdim * es;
+            HY_TRY(dev_alloc(p, (char **)&r.kpool, kb, true));
+            HY_TRY(dev_alloc(p, (char **)&r.vpool, vb, true));
+            e->stats.kv_bytes += kb + vb;
+        } else {
+            const size_t sb = (size_t)c.max_slots * L.heads * L.dim * L.vdim, cb = (size_t)c.max_slots * std::max(1, L.conv_taps - 1) * conv_channels(L);
+            HY_TRY(dev_alloc(p, &r.state, sb, true));
+            HY_TRY(dev_alloc(p, &r.conv_state, cb, true));
+            e->stats.state_bytes += (sb + cb) * 4;
+        }
+    }
+    e->pool = std::make_unique<PagePool>(c.num_pages, c.page_size, c.max_slots, c.max_pages_per_seq);
+    const int R = c.max_rows, W = c.width;
+    e->ld_proj = (max_in + 7) / 8 * 8;
+    e->ld_cat = (max_cat + 7) / 8 * 8;
+    HY_TRY(dev_alloc(p, &e->x, (size_t)R * W));
+    HY_TRY(dev_alloc(p, &e->x0, (size_t)R * W));
+    HY_TRY(dev_alloc(p, &e->proj, (size_t)R * e->ld_proj));
+    HY_TRY(dev_alloc(p, &e->qbuf, (size_t)R * std::max(1, max_q)));
+    HY_TRY(dev_alloc(p, &e->conv_out, (size_t)R * std::max(1, max_c)));
+    HY_TRY(dev_alloc(p, &e->obuf, (size_t)R * std::max(1, max_hv)));
+    HY_TRY(dev_alloc(p, &e->logits, (size_t)R * c.vocab));
+    HY_TRY(dev_alloc(p, (char **)&e->h, (size_t)R * W * es));
+    HY_TRY(dev_alloc(p, (char **)&e->hsel, (size_t)R * W * es));
+    HY_TRY(dev_alloc(p, (char **)&e->cat, (size_t)R * e->ld_cat * es, true));
+    HY_TRY(dev_alloc(p, (char **)&e->cat2, (size_t)R * 2 * W * es));
+    e->stats.workspace_bytes = (size_t)R * (2 * W + e->ld_proj + max_q + max_c + max_hv + c.vocab) * 4 + (size_t)R * (4 * W + e->ld_cat) * es;
+    const size_t mi = meta_ints(R, c.max_slots);
+    HY_TRY(dev_alloc(p, &e->meta_dev, mi));
+    HY_TRY(dev_alloc(p, &e->dmeta_dev, mi, true));
+    HY_HIP(hipHostMalloc((void **)&e->meta_host, mi * 4, hipHostMallocDefault));
+    e->meta = carve(e->meta_dev, R, c.max_slots);
+    e->dmeta = carve(e->dmeta_dev, R, c.max_slots);
+    HY_TRY(dev_alloc(p, &e->table_dev, (size_t)c.max_slots * c.max_pages_per_seq));
+    HY_TRY(dev_alloc(p, &e->ctx_dev, (size_t)c.max_slots, true));
+    HY_TRY(dev_alloc(p, &e->pending_dev, (size_t)c.max_slots, true));
+    HY_TRY(dev_alloc(p, &e->argmax_dev, (size_t)R, true));
+    e->stats.layer_runs = (int)e->runs.size();
+    HY_HIP(hipDeviceSynchronize());
+    *out = e.release();
+    return TL_OK;
+}
+
+extern "C" void tl_hybrid_destroy(tl_hybrid *e) {
+    if (!e) return;
+    (void)hipStreamSynchronize(e->stream);
+    for (auto &g : e->graphs) (void)hipGraphExecDestroy(g.second);
+    for (void *p : e->allocs) (void)hipFree(p);
+    if (e->meta_host) (void)hipHostFree(e->meta_host);
+    if (e->trace_buf) (void)hipFree(e->trace_buf);
+    if (e->owns_stream) (void)hipStreamDestroy(e->stream);
+    delete e;
+}
+
+extern "C" int tl_hybrid_synchronize(tl_hybrid *e) {
+    TL_REQUIRE(e, "hybrid: null engine");
+    HY_HIP(hipStreamSynchronize(e->stream));
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_begin(tl_hybrid *e, int slot) {
+    TL_REQUIRE(e, "hybrid: null engine");
+    TL_REQUIRE(slot >= 0 && slot < e->cfg.max_slots, "hybrid_begin: slot out of range");
+    TL_REQUIRE(!e->pool->live(slot), "hybrid_begin: slot is live");
+    e->pool->begin(slot);
+    for (Run &r : e->runs) {  // the slot's recurrent state starts at zero (fill kernels: a caller may have a capture open on this stream)
+        const tl_hybrid_layer &L = e->layers[r.layer];
+        if (L.kind != TL_MIX_DELTA) continue;
+        const size_t sn = (size_t)L.heads * L.dim * L.vdim, cn = (size_t)std::max(1, L.conv_taps - 1) * conv_channels(L);
+        hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<size_t>(1024, (sn + 255) / 256)), dim3(256), 0, e->stream, r.state + slot * sn, sn, 0.f);
+        hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<size_t>(1024, (cn + 255) / 256)), dim3(256), 0, e->stream, r.conv_state + slot * cn, cn, 0.f);
+        TL_CHECK_LAUNCH("hybrid_begin: state fill");
+    }
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_release(tl_hybrid *e, int slot) {
+    TL_REQUIRE(e, "hybrid: null engine");
+    TL_REQUIRE(slot >= 0 && slot < e->cfg.max_slots, "hybrid_release: slot out of range");
+    TL_REQUIRE(e->pool->live(slot), "hybrid_release: slot holds no sequence");
+    e->pool->release(slot);
+    e->table_dirty = true;
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_move(tl_hybrid *e, int src, int dst) {
+    TL_REQUIRE(e, "hybrid: null engine");
+    TL_REQUIRE(src >= 0 && src < e->cfg.max_slots && dst >= 0 && dst < e->cfg.max_slots && src != dst, "hybrid_move: slot out of range");
+    TL_REQUIRE(e->pool->live(src) && !e->pool->live(dst), "hybrid_move: src must hold a sequence and dst must be free");
+    for (Run &r : e->runs) {  // recurrent state and convolution inputs travel with the sequence; K/V pages stay where they are
+        const tl_hybrid_layer &L = e->layers[r.layer];
+        if (L.kind != TL_MIX_DELTA) continue;
+        const size_t sn = (size_t)L.heads * L.dim * L.vdim, cn = (size_t)std::max(1, L.conv_taps - 1) * conv_channels(L);
+        HY_HIP(hipMemcpyAsync(r.state + dst * sn, r.state + src * sn, sn * 4, hipMemcpyDeviceToDevice, e->stream));
+        HY_HIP(hipMemcpyAsync(r.conv_state + dst * cn, r.conv_state + src * cn, cn * 4, hipMemcpyDeviceToDevice, e->stream));
+    }
+    int32_t tok = 0;
+    HY_HIP(hipMemcpyAsync(&tok, e->pending_dev + src, 4, hipMemcpyDeviceToHost, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    HY_HIP(hipMemcpyAsync(e->pending_dev + dst, &tok, 4, hipMemcpyHostToDevice, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    e->pool->move(src, dst);
+    e->table_dirty = true;
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_context_len(const tl_hybrid *e, int slot) {
+    if (!e || slot < 0 || slot >= e->cfg.max_slots || !e->pool->live(slot)) return -1;
+    return e->pool->context(slot);
+}
+
+extern "C" int tl_hybrid_step(tl_hybrid *e, int n_seqs, const int *slots, const int32_t *tokens, const int *lens, int n_want, const int *want_rows) {
+    TL_REQUIRE(e && slots && tokens && lens, "hybrid_step: null argument");
+    HY_TRY(check_slots(e, n_seqs, slots));
+    const tl_hybrid_config &c = e->cfg;
+    long rows = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        TL_REQUIRE(lens[i] >= 1, "hybrid_step: every chunk holds at least one token");
+        rows += lens[i];
+    }
+    TL_REQUIRE(rows <= c.max_rows, "hybrid_step: more rows than max_rows");
+    TL_REQUIRE(n_want >= 0 && n_want <= c.max_rows && (n_want == 0 || want_rows), "hybrid_step: wanted rows out of range");
+    for (int j = 0; j < n_want; ++j) TL_REQUIRE(want_rows[j] >= 0 && want_rows[j] < rows, "hybrid_step: wanted row outside the step");
+    for (long t = 0; t < rows; ++t) TL_REQUIRE(tokens[t] >= 0 && tokens[t] < c.vocab, "hybrid_step: token id outside the vocabulary");
+    HY_TRY(reserve_all(e, n_seqs, slots, lens));
+    HY_HIP(hipStreamSynchronize(e->stream));  // the pinned staging below may still be read by the previous step's copy
+    const int R = c.max_rows, S = c.max_slots;
+    Meta hm = carve(e->meta_host, R, S);
+    int r = 0;
+    std::vector<int> slot_of_row(rows);
+    for (int i = 0; i < n_seqs; ++i) {
+        hm.seq_row0[i] = r;
+        hm.seq_slot[i] = slots[i];
+        const int ctx = e->pool->context(slots[i]);
+        for (int k = 0; k < lens[i]; ++k, ++r) {
+            hm.tokens[r] = tokens[r];
+            hm.row_seq[r] = i;
+            hm.row_pos[r] = ctx + k;
+            slot_of_row[r] = slots[i];
+        }
+    }
+    hm.seq_row0[n_seqs] = r;
+    for (int j = 0; j < n_want; ++j) {
+        hm.want_rows[j] = want_rows[j];
+        hm.want_slot[j] = slot_of_row[want_rows[j]];
+    }
+    HY_HIP(hipMemcpyAsync(e->meta_dev, e->meta_host, meta_ints(R, S) * 4, hipMemcpyHostToDevice, e->stream));
+    HY_TRY(sync_table(e));
+    HY_TRY(forward(e, e->meta, (int)rows, n_seqs));
+    HY_TRY(head(e, e->meta, n_want, true));
+    for (int i = 0; i < n_seqs; ++i) e->pool->advance(slots[i], lens[i]);
+    e->last_rows = n_want;
+    e->trace_rows = (int)rows;
+    e->stats.steps++;
+    e->stats.rows += rows;
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_set_token(tl_hybrid *e, int slot, int32_t token) {
+    TL_REQUIRE(e, "hybrid: null engine");
+    TL_REQUIRE(slot >= 0 && slot < e->cfg.max_slots && e->pool->live(slot), "hybrid_set_token: slot holds no sequence");
+    TL_REQUIRE(token >= 0 && token < e->cfg.vocab, "hybrid_set_token: token id outside the vocabulary");
+    HY_HIP(hipMemcpyAsync(e->pending_dev + slot, &token, 4, hipMemcpyHostToDevice, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_decode(tl_hybrid *e, int n_seqs, const int *slots, int steps, int use_graph) {
+    TL_REQUIRE(e && slots, "hybrid_decode: null argument");
+    TL_REQUIRE(steps >= 1, "hybrid_decode: steps must be positive");
+    HY_TRY(check_slots(e, n_seqs, slots));
+    const tl_hybrid_config &c = e->cfg;
+    TL_REQUIRE(n_seqs <= c.max_rows, "hybrid_decode: more sequences than max_rows");
+    std::vector<int> extra(n_seqs, steps);
+    HY_TRY(reserve_all(e, n_seqs, slots, extra.data()));
+    const std::vector<int> key(slots, slots + n_seqs);
+    HY_HIP(hipStreamSynchronize(e->stream));
+    const int R = c.max_rows, S = c.max_slots;
+    if (e->dmeta_slots != key) {  // static part of the decode metadata: row i <-> sequence i <-> slots[i]
+        Meta hm = carve(e->meta_host, R, S);
+        std::memset(e->meta_host, 0, meta_ints(R, S) * 4);
+        for (int i = 0; i < n_seqs; ++i) {
+            hm.row_seq[i] = i;
+            hm.seq_row0[i] = i;
+            hm.seq_slot[i] = slots[i];
+            hm.want_rows[i] = i;
+            hm.want_slot[i] = slots[i];
+        }
+        hm.seq_row0[n_seqs] = n_seqs;
+        HY_HIP(hipMemcpyAsync(e->dmeta_dev, e->meta_host, meta_ints(R, S) * 4, hipMemcpyHostToDevice, e->stream));
+        HY_HIP(hipStreamSynchronize(e->stream));
+        e->dmeta_slots = key;
+    }
+    std::vector<int32_t> ctx(S, 0);
+    for (int s = 0; s < S; ++s) ctx[s] = e->pool->live(s) ? e->pool->context(s) : 0;
+    HY_HIP(hipMemcpyAsync(e->ctx_dev, ctx.data(), S * 4, hipMemcpyHostToDevice, e->stream));
+    HY_TRY(sync_table(e));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    auto one_step = [&]() -> int {
+        hipLaunchKernelGGL(decode_meta_kernel, dim3((n_seqs + 63) / 64), dim3(64), 0, e->stream, e->dmeta.seq_slot, n_seqs, e->pending_dev, e->ctx_dev,
+                           e->dmeta.tokens, e->dmeta.row_pos, 0);
+        TL_CHECK_LAUNCH("hybrid decode meta");
+        HY_TRY(forward(e, e->dmeta, n_seqs, n_seqs));
+        HY_TRY(head(e, e->dmeta, n_seqs, true));
+        hipLaunchKernelGGL(decode_meta_kernel, dim3((n_seqs + 63) / 64), dim3(64), 0, e->stream, e->dmeta.seq_slot, n_seqs, e->pending_dev, e->ctx_dev,
+                           e->dmeta.tokens, e->dmeta.row_pos, 1);
+        TL_CHECK_LAUNCH("hybrid decode advance");
+        return TL_OK;
+    };
+    const bool graph = use_graph && !e->trace;
+    if (graph) {
+        auto it = e->graphs.find(key);
+        if (it == e->graphs.end()) {
+            if (e->graphs.size() >= 32) {
+                for (auto &g : e->graphs) (void)hipGraphExecDestroy(g.second);
+                e->graphs.clear();
+            }
+            hipGraph_t g = nullptr;
+            HY_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
+            const int s = one_step();
+            const hipError_t ce = hipStreamEndCapture(e->stream, &g);
+            if (s != 0) {
+                if (g) (void)hipGraphDestroy(g);
+                return s;
+            }
+            HY_HIP(ce);
+            hipGraphExec_t ex = nullptr;
+            HY_HIP(hipGraphInstantiate(&ex, g, nullptr, nullptr, 0));
+            (void)hipGraphDestroy(g);
+            it = e->graphs.emplace(key, ex).first;
+            e->stats.graph_captures++;
+        }
+        for (int k = 0; k < steps; ++k) {
+            HY_HIP(hipGraphLaunch(it->second, e->stream));
+            e->stats.graph_replays++;
+        }
+    } else {
+        for (int k = 0; k < steps; ++k) HY_TRY(one_step());
+    }
+    for (int i = 0; i < n_seqs; ++i) e->pool->advance(slots[i], steps);
+    e->last_rows = n_seqs;
+    e->trace_rows = n_seqs;
+    e->stats.steps += steps;
+    e->stats.rows += (long)steps * n_seqs;
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_read_pending(tl_hybrid *e, int n, const int *slots, int32_t *out) {
+    TL_REQUIRE(e && slots && out, "hybrid_read_pending: null argument");
+    std::vector<int32_t> all(e->cfg.max_slots);
+    HY_HIP(hipMemcpyAsync(all.data(), e->pending_dev, all.size() * 4, hipMemcpyDeviceToHost, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    for (int i = 0; i < n; ++i) {
+        TL_REQUIRE(slots[i] >= 0 && slots[i] < e->cfg.max_slots, "hybrid_read_pending: slot out of range");
+        out[i] = all[slots[i]];
+    }
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_copy_logits(tl_hybrid *e, void *dst_dev, int rows) {
+    TL_REQUIRE(e && dst_dev, "hybrid_copy_logits: null argument");
+    TL_REQUIRE(rows >= 0 && rows <= e->last_rows, "hybrid_copy_logits: more rows than the last step produced");
+    if (rows) HY_HIP(hipMemcpyAsync(dst_dev, e->logits, (size_t)rows * e->cfg.vocab * 4, hipMemcpyDeviceToDevice, e->stream));
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_read_logits(tl_hybrid *e, float *dst_host, int rows) {
+    TL_REQUIRE(e && dst_host, "hybrid_read_logits: null argument");
+    TL_REQUIRE(rows >= 0 && rows <= e->last_rows, "hybrid_read_logits: more rows than the last step produced");
+    if (rows) HY_HIP(hipMemcpyAsync(dst_host, e->logits, (size_t)rows * e->cfg.vocab * 4, hipMemcpyDeviceToHost, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_read_argmax(tl_hybrid *e, int rows, int32_t *out) {
+    TL_REQUIRE(e && out, "hybrid_read_argmax: null argument");
+    TL_REQUIRE(rows >= 0 && rows <= e->last_rows, "hybrid_read_argmax: more rows than the last step produced");
+    if (rows) HY_HIP(hipMemcpyAsync(out, e->argmax_dev, (size_t)rows * 4, hipMemcpyDeviceToHost, e->stream));
+    HY_HIP(hipStreamSynchronize(e->stream));
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_set_trace(tl_hybrid *e, int on) {
+    TL_REQUIRE(e, "hybrid: null engine");
+    if (on && !e->trace_buf) HY_HIP(hipMalloc((void **)&e->trace_buf, e->runs.size() * (size_t)e->cfg.max_rows * e->cfg.width * 4));
+    e->trace = on != 0;
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_read_trace(tl_hybrid *e, int run, float *dst_host, int rows) {
+    TL_REQUIRE(e && dst_host && e->trace_buf, "hybrid_read_trace: tracing is off");
+    TL_REQUIRE(run >= 0 && run < (int)e->runs.size() && rows >= 0 && rows <= e->trace_rows, "hybrid_read_trace: run or rows out of range");
+    HY_HIP(hipStreamSynchronize(e->stream));
+    HY_HIP(hipMemcpy(dst_host, e->trace_buf + (size_t)run * e->cfg.max_rows * e->cfg.width, (size_t)rows * e->cfg.width * 4, hipMemcpyDeviceToHost));
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_get_stats(const tl_hybrid *e, tl_hybrid_stats *out) {
+    TL_REQUIRE(e && out, "hybrid_get_stats: null argument");
+    tl_hybrid_stats s = e->stats;
+    const PagePoolStats &p = e->pool->stats();
+    s.pages_in_use = p.pages_in_use;
+    s.pages_free = e->pool->free_pages();
+    s.peak_pages_in_use = p.peak_pages_in_use;
+    s.page_allocations = p.page_allocations;
+    s.reused_page_allocations = p.reused_page_allocations;
+    s.slot_begins = p.slot_begins;
+    s.reused_slot_begins = p.reused_slot_begins;
+    *out = s;
+    return TL_OK;
+}
+
+extern "C" int tl_hybrid_linear(int dtype, const void *a_dev, int lda, const void *w_dev, float *out_dev, int ldc, int M, int N, int K, int force_kernel,
+                                void *stream) {
+    TL_REQUIRE(a_dev && w_dev && out_dev, "hybrid_linear: null argument");
+    TL_REQUIRE(dtype == TL_HY_BF16 || dtype == TL_HY_F32, "hybrid_linear: dtype must be bfloat16 or float32");
+    TL_REQUIRE(M > 0 && N > 0 && K > 0 && lda >= K && ldc >= N, "hybrid_linear: bad shape");
+    if (dtype == TL_HY_BF16) return linear_t<BF16>(a_dev, lda, w_dev, out_dev, ldc, M, N, K, 0, 1.f, nullptr, force_kernel, (hipStream_t)stream);
+    return linear_t<F32>(a_dev, lda, w_dev, out_dev, ldc, M, N, K, 0, 1.f, nullptr, force_kernel, (hipStream_t)stream);
+}

@@ -1,0 +1,583 @@
+// Kernels of the layer-list engine (include/tinyllm_hybrid.h).  D = F32 or BF16 (common.h): the type of matrices, of
+// activations entering a matrix product and of K/V pages.  Everything else is float32.
+//
+// Packed rows: a step's tokens lie back to back, sequence after sequence.  Per row: row_seq (index into the step's
+// sequence list) and row_pos (position in its sequence).  Per sequence: seq_row0 (first row; seq_row0[n] = rows),
+// seq_slot (state slot = block-table row).
+#pragma once
+#include "common.h"
+
+namespace tl {
+namespace hy {
+
+template <typename D>
+__device__ __forceinline__ float ld(const typename D::storage *p, size_t i) { return D::to_float(p[i]); }
+
+// generic block reduction (sum), blockDim.x a multiple of 64 and <= 1024; red = 16 floats of LDS
+__device__ __forceinline__ float block_sum(float v, float *red) {
+    v = wave_sum(v);
+    const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += red[i];
+    return t;
+}
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float act_f(float z, int kind) {
+    if (kind == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752440f));
+    if (kind == 1) return 0.5f * z * (1.f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+    return silu_f(z);
+}
+
+// ---- embedding gather: x0 = x = embed[token] -------------------------------------------------------------------
+template <typename D>
+__global__ void embed_kernel(const int32_t *tokens, const typename D::storage *embed, float *x0, float *x, int width, int vocab) {
+    const int t = blockIdx.x;
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float v = ld<D>(embed, (size_t)tok * width + c);
+        x0[(size_t)t * width + c] = v;
+        x[(size_t)t * width + c] = v;
+    }
+}
+
+// ---- RMS norm of float32 rows -> D rows: x / sqrt(mean(x^2) + eps) * (offset + w).  rows_idx: optional gather. ----
+template <typename D>
+__global__ void norm_kernel(const float *x, const float *w, float offset, float eps, typename D::storage *out, int width,
+                            const int32_t *rows_idx) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const float *src = x + (size_t)(rows_idx ? rows_idx[r] : r) * width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) ss += src[c] * src[c];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)r * width + c] = D::from_float(src[c] * inv * (offset + w[c]));
+}
+
+// ---- [x ; x0] as D rows of 2*width (input of the loop-entry projection) ------------------------------------------
+template <typename D>
+__global__ void pack2_kernel(const float *x, const float *x0, typename D::storage *out, int width) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < 2 * width; c += blockDim.x)
+        out[(size_t)t * 2 * width + c] = D::from_float(c < width ? x[(size_t)t * width + c] : x0[(size_t)t * width + c - width]);
+}
+
+// ---- tile matrix product: out[M, N] (+)= A[M, K] . W[N, K]^T, float32 accumulation on the matrix cores ------------
+// 64 x 64 output tile per 256-thread workgroup, 4 waves of 32 x 32 (2 x 2 MFMA 16x16 tiles), K in steps of 32 through LDS.
+// bf16: v_mfma_f32_16x16x32_bf16; fp32: v_mfma_f32_16x16x4_f32 (full fp32 products).  Any M, N, K: edges are zero-filled in LDS.
+// EPI 0: out = acc   1: out += alpha * acc   2: out = acc + bias[n]
+template <typename D, int EPI>
+__global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
+                                                        int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok) {
+    using S = typename D::storage;
+    constexpr bool BF = sizeof(S) == 2;
+    constexpr int KT = 32, LD = BF ? KT + 8 : KT + 1;
+    __shared__ S As[64 * LD];
+    __shared__ S Ws[64 * LD];
+    // XCD-aware tile order: consecutive workgroup ids go to different XCDs (round robin over 8), so give each XCD a contiguous run of tiles
+    const int nt_n = (N + 63) / 64, nt_m = (M + 63) / 64, total = nt_n * nt_m;
+    int id = blockIdx.x;
+    {
+        const int per = (total + 7) / 8, xcd = id & 7, k = id >> 3;
+        const int mapped = xcd * per + k;
+        id = (total % 8 == 0) ? mapped : id;
+    }
+    const int tm = id / nt_n, tn = id % nt_n;
+    const int m0 = tm * 64, n0 = tn * 64;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    f32x4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int lr = tid >> 2, lk = (tid & 3) * 8;  // loader: row of the tile, first of 8 consecutive k
+    for (int k0 = 0; k0 < K; k0 += KT) {
+        __syncthreads();
+        {
+            const int gm = m0 + lr, gn = n0 + lr, gk = k0 + lk;
+            S av[8], wv[8];
+            if (vec_ok && gm < M && gk + 8 <= K) {
+                if constexpr (BF) *reinterpret_cast<u32x4 *>(av) = *reinterpret_cast<const u32x4 *>(A + (size_t)gm * lda + gk);
+                else {
+                    *reinterpret_cast<u32x4 *>(av) = *reinterpret_cast<const u32x4 *>(A + (size_t)gm * lda + gk);
+                    *reinterpret_cast<u32x4 *>(av + 4) = *reinterpret_cast<const u32x4 *>(A + (size_t)gm * lda + gk + 4);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) av[i] = (gm < M && gk + i < K) ? A[(size_t)gm * lda + gk + i] : (S)0;
+            }
+            if (vec_ok && gn < N && gk + 8 <= K) {
+                if constexpr (BF) *reinterpret_cast<u32x4 *>(wv) = *reinterpret_cast<const u32x4 *>(W + (size_t)gn * K + gk);
+                else {
+                    *reinterpret_cast<u32x4 *>(wv) = *reinterpret_cast<const u32x4 *>(W + (size_t)gn * K + gk);
+                    *reinterpret_cast<u32x4 *>(wv + 4) = *reinterpret_cast<const u32x4 *>(W + (size_t)gn * K + gk + 4);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) wv[i] = (gn < N && gk + i < K) ? W[(size_t)gn * K + gk + i] : (S)0;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                As[lr * LD + lk + i] = av[i];
+                Ws[lr * LD + lk + i] = wv[i];
+            }
+        }
+        __syncthreads();
+        if constexpr (BF) {
+            bf16x8_t af[2], bfr[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const S *pa = As + (wm * 32 + i * 16 + (lane & 15)) * LD + (lane >> 4) * 8;
+                const S *pb = Ws + (wn * 32 + i * 16 + (lane & 15)) * LD + (lane >> 4) * 8;
+                u32x4 ua = *reinterpret_cast<const u32x4 *>(pa), ub = *reinterpret_cast<const u32x4 *>(pb);
+                af[i] = __builtin_bit_cast(bf16x8_t, ua);
+                bfr[i] = __builtin_bit_cast(bf16x8_t, ub);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KT; ks += 4) {
+                float a[2], b[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    a[i] = As[(wm * 32 + i * 16 + (lane & 15)) * LD + ks + (lane >> 4)];
+                    b[i] = Ws[(wn * 32 + i * 16 + (lane & 15)) * LD + ks + (lane >> 4)];
+                }
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+    // D layout of the 16x16 MFMA: lane holds column (lane & 15), rows 4 * (lane >> 4) + r
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int gm = m0 + wm * 32 + i * 16 + (lane >> 4) * 4 + r, gn = n0 + wn * 32 + j * 16 + (lane & 15);
+                if (gm < M && gn < N) {
+                    float *o = out + (size_t)gm * ldc + gn;
+                    const float v = acc[i][j][r];
+                    if constexpr (EPI == 0) *o = v;
+                    else if constexpr (EPI == 1) *o += alpha * v;
+                    else *o = v + bias[gn];
+                }
+            }
+}
+
+// ---- row matrix product for a few rows (decode): each wave owns one output column and streams its weight row once ----
+// M <= 8.  Lanes stride over K, 8 elements at a time where the layout allows 16-byte loads.
+template <typename D, int EPI>
+__global__ __launch_bounds__(256) void gemm_rows_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
+                                                        int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok) {
+    using S = typename D::storage;
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    float acc[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) acc[m] = 0.f;
+    const S *wrow = W + (size_t)n * K;
+    if (vec_ok) {
+        for (int k = lane * 8; k + 8 <= K; k += 64 * 8) {
+            float wf[8];
+            if constexpr (sizeof(S) == 2) {
+                u32x4 u = *reinterpret_cast<const u32x4 *>(wrow + k);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    wf[2 * i] = __uint_as_float(u[i] << 16);
+                    wf[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) wf[i] = D::to_float(wrow[k + i]);
+            }
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                if (m < M) {
+                    const S *arow = A + (size_t)m * lda + k;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[m] += wf[i] * D::to_float(arow[i]);
+                }
+            }
+        }
+        for (int k = (K / 8) * 8 + lane; k < K; k += 64) {
+            const float wf = D::to_float(wrow[k]);
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+                if (m < M) acc[m] += wf * D::to_float(A[(size_t)m * lda + k]);
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) {
+            const float wf = D::to_float(wrow[k]);
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+                if (m < M) acc[m] += wf * D::to_float(A[(size_t)m * lda + k]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+        if (m < M) {  // M is uniform over the grid
+            const float v = wave_sum(acc[m]);
+            if (lane == 0) {
+                float *o = out + (size_t)m * ldc + n;
+                if constexpr (EPI == 0) *o = v;
+                else if constexpr (EPI == 1) *o += alpha * v;
+                else *o = v + bias[n];
+            }
+        }
+    }
+}
+
+// ---- attention, step 1: rotary positions + unit-RMS on q and k; k and v rows appended to their pages -----------------
+// proj: [rows, ldp] float32 with q | k | v at columns 0 | H*dim | (H+G)*dim.  One wave per (row, head of q|k|v).
+// Rotation of the pair (2i, 2i+1) by pos * inv_freq[i] for i < rot_dims/2.
+template <typename D>
+__global__ __launch_bounds__(64) void attn_prep_kernel(const float *proj, int ldp, const int32_t *row_seq, const int32_t *row_pos,
+                                                       const int32_t *seq_slot, const int32_t *block_table, int max_pages, int page_size,
+                                                       const float *inv_freq, int rot_dims, int unit_rms, float eps, int H, int G, int dim,
+                                                       int vdim, float *qbuf, typename D::storage *kpool, typename D::storage *vpool) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int pos = row_pos[t], slot = seq_slot[row_seq[t]];
+    const int page = block_table[(size_t)slot * max_pages + pos / page_size], in_page = pos % page_size;
+    if (hh >= H + G) {  // a value head: copy
+        const int g = hh - H - G;
+        const float *src = proj + (size_t)t * ldp + (size_t)(H + G) * dim + (size_t)g * vdim;
+        typename D::storage *dst = vpool + (((size_t)page * G + g) * page_size + in_page) * vdim;
+        for (int c = lane; c < vdim; c += 64) dst[c] = D::from_float(src[c]);
+        return;
+    }
+    const float *src = proj + (size_t)t * ldp + (size_t)hh * dim;
+    // pairs are rotated by the lane that owns the even element; elements beyond rot_dims pass
+    float ss = 0.f;
+    const int npairs = (dim + 1) / 2;
+    const bool is_q = hh < H;
+    float *qdst = qbuf + ((size_t)t * H + hh) * dim;
+    typename D::storage *kdst = is_q ? nullptr : kpool + (((size_t)page * G + (hh - H)) * page_size + in_page) * dim;
+    // pass 1: rotate into registers (at most 8 pairs per lane: dim <= 1024), accumulate the sum of squares
+    float ra[8], rb[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int p = lane + it * 64;
+        ra[it] = rb[it] = 0.f;
+        if (p < npairs) {
+            const int c = 2 * p;
+            float u = src[c], v = (c + 1 < dim) ? src[c + 1] : 0.f;
+            if (c + 1 < rot_dims) {
+                const float a = (float)pos * inv_freq[p];
+                float sn, cs;
+                sincosf(a, &sn, &cs);
+                const float nu = u * cs - v * sn, nv = v * cs + u * sn;
+                u = nu;
+                v = nv;
+            }
+            ra[it] = u;
+            rb[it] = v;
+            ss += u * u + v * v;
+        }
+    }
+    ss = wave_sum(ss);
+    const float inv = unit_rms ? 1.f / sqrtf(ss / (float)dim + eps) : 1.f;
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const int p = lane + it * 64;
+        if (p < npairs) {
+            const int c = 2 * p;
+            if (is_q) {
+                qdst[c] = ra[it] * inv;
+                if (c + 1 < dim) qdst[c + 1] = rb[it] * inv;
+            } else {
+                kdst[c] = D::from_float(ra[it] * inv);
+                if (c + 1 < dim) kdst[c + 1] = D::from_float(rb[it] * inv);
+            }
+        }
+    }
+}
+
+// ---- attention, step 2 (row form): one wave per (row, query head) walks the keys 0 .. pos of its sequence ---------------
+// float32 scores and weights, running maximum; the sink is the start value of the running pair (max 0, sum 1).
+// out: cat[t, h*vdim + c] = (sum_j p_j v_j[c]) * sigmoid(gate[t, h*vdim + c])   (D rows of ldo)
+template <typename D>
+__global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
+                                                       const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
+                                                       const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
+                                                       float scale, int sink, const float *gate, int ldg, typename D::storage *out, int ldo) {
+    extern __shared__ float smem[];
+    float *qs = smem;        // [dim]
+    float *ps = smem + dim;  // [64]
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int pos = row_pos[t], slot = seq_slot[row_seq[t]], g = h / (H / G);
+    const int32_t *bt = block_table + (size_t)slot * max_pages;
+    for (int c = lane; c < dim; c += 64) qs[c] = qbuf[((size_t)t * H + h) * dim + c];
+    __syncthreads();
+    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};  // vdim <= 256
+    for (int kb = 0; kb <= pos; kb += 64) {
+        const int j = kb + lane;
+        float s = -INFINITY;
+        if (j <= pos) {
+            const typename D::storage *kr = kpool + (((size_t)bt[j / page_size] * G + g) * page_size + j % page_size) * dim;
+            float d = 0.f;
+            for (int c = 0; c < dim; ++c) d += qs[c] * D::to_float(kr[c]);
+            s = d * scale;
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float p = (j <= pos) ? expf(s - m_new) : 0.f;
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        l = l * corr + wave_sum(p);
+        m = m_new;
+        __syncthreads();
+        ps[lane] = p;
+        __syncthreads();
+        const int cnt = min(64, pos - kb + 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] *= corr;
+        for (int jj = 0; jj < cnt; ++jj) {
+            const int jg = kb + jj;
+            const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * G + g) * page_size + jg % page_size) * vdim;
+            const float pj = ps[jj];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = lane + i * 64;
+                if (c < vdim) acc[i] += pj * D::to_float(vr[c]);
+            }
+        }
+    }
+    const float invl = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + i * 64;
+        if (c < vdim) {
+            float o = acc[i] * invl;
+            if (gate) o *= sigmoid_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]);
+            out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o);
+        }
+    }
+}
+
+// ---- feed-forward activation: cat[t, col0 + c] = act(proj[t, up0 + c]) ---------------------------------------------------
+template <typename D>
+__global__ void ff_act_kernel(const float *proj, int ldp, int up0, int ff, int kind, typename D::storage *out, int ldo, int col0, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * ff) return;
+    const int t = (int)(i / ff), c = (int)(i % ff);
+    out[(size_t)t * ldo + col0 + c] = D::from_float(act_f(proj[(size_t)t * ldp + up0 + c], kind));
+}
+
+// ---- short causal depthwise convolution + SiLU over the first C columns of proj -------------------------------------------
+// state: [slots, taps-1, C] float32 = the last taps-1 inputs of the sequence, oldest first (zeros at its start).
+__global__ void conv_kernel(const float *proj, int ldp, const float *w, int taps, int C, const int32_t *row_seq, const int32_t *seq_row0,
+                            const int32_t *seq_slot, const float *state, float *out, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * C) return;
+    const int t = (int)(i / C), c = (int)(i % C);
+    const int s = row_seq[t], r0 = seq_row0[s], li = t - r0;
+    const float *st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int idx = li - (taps - 1) + j;
+        const float v = idx >= 0 ? proj[(size_t)(r0 + idx) * ldp + c] : st[(size_t)(taps - 1 + idx) * C + c];
+        acc += w[(size_t)c * taps + j] * v;
+    }
+    out[(size_t)t * C + c] = silu_f(acc);
+}
+// the convolution's inputs move on: the last taps-1 inputs after this chunk.  One thread per (sequence, channel).
+__global__ void conv_state_kernel(const float *proj, int ldp, int taps, int C, const int32_t *seq_row0, const int32_t *seq_slot, float *state,
+                                  int n_seqs) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)n_seqs * C) return;
+    const int s = (int)(i / C), c = (int)(i % C);
+    const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0;
+    float *st = state + (size_t)seq_slot[s] * (taps - 1) * C;
+    for (int j = 0; j < taps - 1; ++j) {  // ascending: st[j + n] is read before it is written
+        const int src = n - (taps - 1) + j;
+        st[(size_t)j * C + c] = src >= 0 ? proj[(size_t)(r0 + src) * ldp + c] : st[(size_t)(j + n) * C + c];
+    }
+}
+
+// ---- gated delta rule, token by token ------------------------------------------------------------------------------------
+// grid (heads, sequences, column blocks of VB).  A thread holds RPT rows of one state column in registers; R = lanes per column
+// (a power of two <= 64, adjacent lanes), so key_dim <= RPT * R.  Per token:  S *= g;  u = beta (v - S^T k);  S += k u^T;  o = S^T q.
+// qkv: [rows, C] float32 after convolution + SiLU, q | k | v at 0 | G*dim | 2*G*dim.  q and k become unit vectors here
+// (x / sqrt(sum x^2 + unit_eps); q also * dim^-1/2).  ab: proj columns a0 + h (decay input) and b0 + h (beta input).
+template <int RPT>
+__global__ void delta_kernel(const float *qkv, int C, const float *proj, int ldp, int a0, int b0, const float *a_log, const float *dt_bias,
+                             float unit_eps, const int32_t *seq_row0, const int32_t *seq_slot, float *state, float *obuf, int H, int G, int dim,
+                             int vdim, int R, int VB, int TB) {
+    extern __shared__ float smem[];
+    float *qs = smem;                 // [TB, dim]
+    float *ks = qs + (size_t)TB * dim;  // [TB, dim]
+    float *vs = ks + (size_t)TB * dim;  // [TB, VB]
+    float *gs = vs + (size_t)TB * VB;   // [TB]
+    float *bs = gs + TB;              // [TB]
+    const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * VB;
+    const int kh = h / (H / G);
+    const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int jl = tid / R, r = tid % R, j = j0 + jl;
+    const bool active = jl < VB && j < vdim;
+    float S[RPT];
+    float *sp = state + (((size_t)slot * H + h) * dim) * vdim;  // [dim, vdim]
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+        const int d = r * RPT + i;
+        S[i] = (active && d < dim) ? sp[(size_t)d * vdim + j] : 0.f;
+    }
+    const float decay_rate = -expf(a_log[h]), bias = dt_bias[h], qscale = 1.f / sqrtf((float)dim);
+    for (int t0 = 0; t0 < n; t0 += TB) {
+        const int nt = min(TB, n - t0);
+        __syncthreads();
+        for (int i = tid; i < nt * dim; i += blockDim.x) {
+            const int tt = i / dim, d = i % dim;
+            const float *row = qkv + (size_t)(r0 + t0 + tt) * C;
+            qs[i] = row[(size_t)kh * dim + d];
+            ks[i] = row[(size_t)(G + kh) * dim + d];
+        }
+        for (int i = tid; i < nt * VB; i += blockDim.x) {
+            const int tt = i / VB, c = i % VB;
+            vs[i] = (j0 + c < vdim) ? qkv[(size_t)(r0 + t0 + tt) * C + (size_t)2 * G * dim + (size_t)h * vdim + j0 + c] : 0.f;
+        }
+        for (int tt = tid; tt < nt; tt += blockDim.x) {
+            const float *prow = proj + (size_t)(r0 + t0 + tt) * ldp;
+            gs[tt] = expf(decay_rate * softplus_f(prow[a0 + h] + bias));
+            bs[tt] = sigmoid_f(prow[b0 + h]);
+        }
+        __syncthreads();
+        for (int tt = wave; tt < nt; tt += nwaves) {  // unit vectors: one wave per token
+            float sq = 0.f, sk = 0.f;
+            for (int d = lane; d < dim; d += 64) {
+                sq += qs[tt * dim + d] * qs[tt * dim + d];
+                sk += ks[tt * dim + d] * ks[tt * dim + d];
+            }
+            sq = wave_sum(sq);
+            sk = wave_sum(sk);
+            const float iq = qscale / sqrtf(sq + unit_eps), ik = 1.f / sqrtf(sk + unit_eps);
+            for (int d = lane; d < dim; d += 64) {
+                qs[tt * dim + d] *= iq;
+                ks[tt * dim + d] *= ik;
+            }
+        }
+        __syncthreads();
+        if (active) {
+            for (int tt = 0; tt < nt; ++tt) {
+                const float g = gs[tt], b = bs[tt];
+                const float *kt = ks + tt * dim + r * RPT, *qt = qs + tt * dim + r * RPT;
+                float kv[RPT];
+                float dot = 0.f;
+#pragma unroll
+                for (int i = 0; i < RPT; ++i) {
+                    kv[i] = (r * RPT + i < dim) ? kt[i] : 0.f;
+                    S[i] *= g;
+                    dot += S[i] * kv[i];
+                }
+                for (int o = 1; o < R; o <<= 1) dot += __shfl_xor(dot, o, 64);
+                const float u = b * (vs[tt * VB + jl] - dot);
+                float od = 0.f;
+#pragma unroll
+                for (int i = 0; i < RPT; ++i) {
+                    S[i] += kv[i] * u;
+                    od += S[i] * ((r * RPT + i < dim) ? qt[i] : 0.f);
+                }
+                for (int o = 1; o < R; o <<= 1) od += __shfl_xor(od, o, 64);
+                if (r == 0) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
+            }
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+            const int d = r * RPT + i;
+            if (d < dim) sp[(size_t)d * vdim + j] = S[i];
+        }
+    }
+}
+
+// ---- read-out of the delta rule: per (row, head) o / rms(o) * w * silu(gate) -> cat columns h*vdim .. ----------------------
+template <typename D>
+__global__ __launch_bounds__(64) void delta_out_kernel(const float *obuf, const float *w, float eps, const float *gate, int ldg, int H, int vdim,
+                                                       typename D::storage *out, int ldo) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float *o = obuf + ((size_t)t * H + h) * vdim;
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += 64) ss += o[c] * o[c];
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
+    for (int c = lane; c < vdim; c += 64)
+        out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o[c] * inv * w[c] * silu_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]));
+}
+
+// ---- small helpers -----------------------------------------------------------------------------------------------------------
+__global__ void add_rowvec_kernel(float *x, const float *v, int width, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < (size_t)rows * width) x[i] += v[i % width];
+}
+__global__ void fill_kernel(float *p, size_t n, float v) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+// argmax of each logits row (first index wins on ties); also the next input token of the row's slot when slot_of_row is given
+__global__ __launch_bounds__(256) void argmax_kernel(const float *logits, int vocab, int32_t *out, const int32_t *slot_of_row, int32_t *pending) {
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    const int r = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+    const float *row = logits + (size_t)r * vocab;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int c = tid; c < vocab; c += 256) {
+        const float v = row[c];
+        if (v > best || (v == best && c < idx)) {
+            best = v;
+            idx = c;
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(idx, o, 64);
+        if (ov > best || (ov == best && oi < idx)) {
+            best = ov;
+            idx = oi;
+        }
+    }
+    if (lane == 0) {
+        bv[tid >> 6] = best;
+        bi[tid >> 6] = idx;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
+                best = bv[w];
+                idx = bi[w];
+            }
+        if (idx == 0x7fffffff) idx = 0;
+        out[r] = idx;
+        if (slot_of_row) pending[slot_of_row[r]] = idx;
+    }
+}
+// decode bookkeeping on the device: the step's rows are one token per listed slot; tokens come from `pending`, positions from `ctx`
+__global__ void decode_meta_kernel(const int32_t *slots, int n, const int32_t *pending, int32_t *ctx, int32_t *tokens, int32_t *row_pos,
+                                   int advance) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int s = slots[i];
+    if (advance) ctx[s] += 1;
+    else {
+        tokens[i] = pending[s];
+        row_pos[i] = ctx[s];
+    }
+}
+
+}  // namespace hy
+}  // namespace tl

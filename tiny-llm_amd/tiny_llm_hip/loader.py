@@ -92,10 +92,38 @@ def _quantization(config: dict) -> tuple[int, int]:
     return group_size, bits
 
 
-def load_weights(model_dir: str | Path, device: str = "cuda") -> SimpleNamespace:
-    """The mlx_lm-shaped model object of an MLX 4-bit Qwen3 checkpoint directory (see module docstring)."""
+def _load_layer_list(model_dir: Path, config: dict, dtype: torch.dtype | None) -> SimpleNamespace:
+    """A layer-list checkpoint (layer_list.FAMILIES by config.json's ``architecture``): unquantised tensors by name, checked against
+    the family's table of names and shapes.  Tensors stay on the host here; the engine packs them into its own layout on the device."""
+    from .layer_list import FAMILIES
+
+    read_config, tensor_shapes = FAMILIES[config["architecture"]]
+    cfg = read_config(config)
+    src = _TensorSource(model_dir)
+    tensors = {}
+    for name, shape in tensor_shapes(cfg).items():
+        t = src.get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: expected shape {tuple(shape)}, found {tuple(t.shape)}")
+        if not t.dtype.is_floating_point:
+            raise ValueError(f"{name}: expected a floating-point tensor, found {t.dtype}")
+        tensors[name] = t
+    args = SimpleNamespace(vocab_size=cfg.vocab, hidden_size=cfg.width, num_hidden_layers=len(cfg.layers), architecture=cfg.family)
+    return SimpleNamespace(family=cfg.family, config=cfg, tensors=tensors, dtype=dtype or torch.bfloat16, args=args)
+
+
+def load_weights(model_dir: str | Path, device: str = "cuda", dtype: torch.dtype | None = None) -> SimpleNamespace:
+    """The model object of a checkpoint directory: the mlx_lm-shaped tree of an MLX 4-bit Qwen3 checkpoint (see module docstring), or,
+    where config.json names a layer-list architecture, that family's description and tensors (``dtype``: torch.bfloat16 or
+    torch.float32, the precision the engine will run in)."""
     model_dir = Path(model_dir)
     config = json.loads((model_dir / "config.json").read_text())
+    from .layer_list import FAMILIES
+
+    if config.get("architecture") in FAMILIES:
+        return _load_layer_list(model_dir, config, dtype)
+    if dtype not in (None, torch.bfloat16):
+        raise ValueError("the W4A16 path runs in bfloat16 only")
     missing = [k for k in _CONFIG_KEYS if k not in config]
     if missing:
         raise ValueError(f"config.json lacks {missing}")
@@ -277,6 +305,8 @@ def load(name_or_path: str, device: str = "cuda"):
     """(model, tokenizer) like ``mlx_lm.load``; see the module docstring."""
     model_dir = resolve_model_dir(name_or_path)
     model = load_weights(model_dir, device=device)
+    if getattr(model, "family", None) and not any((model_dir / f).is_file() for f in ("tokenizer.json", "tokenizer_config.json")):
+        return model, None  # a layer-list checkpoint without tokenizer files: token ids in, token ids out
     from transformers import AutoTokenizer
 
     hf_tok = AutoTokenizer.from_pretrained(str(model_dir), local_files_only=True)

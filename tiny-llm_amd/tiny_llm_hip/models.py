@@ -21,3 +21,18 @@ def dispatch_model(model_name: str, mlx_model, week: int, **kwargs):
         if fused_engine_requested():  # TINY_LLM_FUSED_ENGINE=1: the same call surface on the fused decode engine
             return Qwen3ModelFused(mlx_model, **kwargs)
     return cls(mlx_model, **kwargs)
+
+
+def engine_for(model, **kwargs):
+    """The serving engine of a loaded checkpoint (loader.load / load_weights), chosen by what the checkpoint is: a layer-list family
+    (config.json ``architecture`` in layer_list.FAMILIES) runs on the layer-list engine, an MLX 4-bit Qwen3 tree on the fused W4A16
+    decode engine.  Both have the same request-level surface (begin / prefill / decode / release ...); keyword arguments are the pool
+    sizes (page_size, num_pages, max_batch, max_pages_per_seq, max_prefill_rows)."""
+    if getattr(model, "family", None) is not None:
+        from .hybrid_engine import HybridEngine
+
+        return HybridEngine(model, **kwargs)
+    from .engine import DecodeEngine
+
+    kwargs.pop("dtype", None)
+    return DecodeEngine(model, **kwargs)
