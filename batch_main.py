@@ -30,32 +30,40 @@ def main(argv=None):
     args = ap.parse_args(argv)
 
     from tiny_llm_hip import load
-    from tiny_llm_hip.engine import DecodeEngine, batch_generate_ids
+    from tiny_llm_hip.engine import batch_generate_ids
+    from tiny_llm_hip.models import engine_for
     from main import chat_prompt
 
     model, tokenizer = load(args.model)
     prompts = [l for l in Path(args.prompts_file).read_text().splitlines() if l.strip()] if args.prompts_file else DEFAULT_PROMPTS
+    if tokenizer is None and not args.prompts_file:
+        raise ValueError("this checkpoint has no tokenizer: give --prompts-file with one prompt of token ids per line")
     encoded, limits = [], []
     for text in prompts:
-        full = text if args.raw_prompts else chat_prompt(tokenizer, text, args.enable_thinking)
-        ids = tokenizer.encode(full, add_special_tokens=False)
+        if tokenizer is None:  # a layer-list checkpoint without tokenizer files: token ids in, token ids out
+            ids = [int(t) for t in text.replace(",", " ").split()]
+        else:
+            full = text if args.raw_prompts else chat_prompt(tokenizer, text, args.enable_thinking)
+            ids = tokenizer.encode(full, add_special_tokens=False)
         if len(ids) >= args.max_seq_len:
             raise ValueError(f"prompt of {len(ids)} tokens exceeds max_seq_len {args.max_seq_len}")
         encoded.append(ids)
         limits.append(args.max_seq_len - len(ids))
     pages_per_seq = args.max_seq_len // 128 + 2
-    engine = DecodeEngine(model, page_size=128, num_pages=pages_per_seq * (args.batch_size + 1) + 2,
-                          max_batch=args.batch_size + 1, max_prefill_rows=args.prefill_step, kv_format=args.kv_format)
+    extra = {} if getattr(model, "family", None) is not None else {"kv_format": args.kv_format}
+    engine = engine_for(model, page_size=128, num_pages=pages_per_seq * (args.batch_size + 1) + 2,
+                        max_batch=args.batch_size + 1, max_prefill_rows=max(args.prefill_step, args.batch_size + 1), **extra)
+    eos = tokenizer.eos_token_id if tokenizer is not None else None
     try:
         done = batch_generate_ids(engine, encoded, limits, batch_size=args.batch_size, prefill_step=args.prefill_step,
-                                  eos_token_id=tokenizer.eos_token_id)
+                                  eos_token_id=eos)
     finally:
         engine.close()
     results = []
     for idx, ids in done:
-        if ids and ids[-1] == tokenizer.eos_token_id:
+        if ids and ids[-1] == eos:
             ids = ids[:-1]
-        text = tokenizer.decode(ids)
+        text = tokenizer.decode(ids) if tokenizer is not None else " ".join(str(t) for t in ids)
         results.append((idx, text))
         print(f"--- {idx} ---\nQ: {prompts[idx]}\nA: {text}")
     return results

@@ -31,6 +31,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--raw-prompt", action="store_true", help="do not wrap the prompt in the chat template")
     ap.add_argument("--max-new-tokens", type=int, default=256)
     ap.add_argument("--proposal-length", type=int, default=4)
+    ap.add_argument("--prompt-ids", default=None, help="the prompt as token ids with commas (checkpoints without a tokenizer); ids are printed")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="layer-list checkpoints: the engine's precision")
     return ap
 
 
@@ -44,7 +46,11 @@ def main(argv=None) -> str:
     args = build_parser().parse_args(argv)
     from tiny_llm_hip import load
 
-    model, tokenizer = load(args.model)
+    import torch
+
+    model, tokenizer = load(args.model, dtype=getattr(torch, args.dtype))
+    if getattr(model, "family", None) is not None:
+        return generate_layer_list(model, tokenizer, args)
     prompt = args.prompt if args.raw_prompt else chat_prompt(tokenizer, args.prompt, args.enable_thinking)
     if args.solution == "ops":
         from tiny_llm_hip import Qwen3ModelWeek3, make_sampler, simple_generate_with_kv_cache, speculative_generate
@@ -85,6 +91,34 @@ def main(argv=None) -> str:
     finally:
         engine.close()
     text = tokenizer.decode(out)
+    print(text)
+    return text
+
+
+def generate_layer_list(model, tokenizer, args) -> str:
+    """A layer-list checkpoint (tiny_llm_hip.layer_list.FAMILIES) on its engine: greedy on the device, or the sampler flags."""
+    import torch
+    from tiny_llm_hip.models import engine_for
+
+    if args.prompt_ids is not None:
+        ids = [int(t) for t in args.prompt_ids.replace(",", " ").split()]
+    elif tokenizer is not None:
+        ids = tokenizer.encode(args.prompt if args.raw_prompt else chat_prompt(tokenizer, args.prompt, args.enable_thinking), add_special_tokens=False)
+    else:
+        raise ValueError("this checkpoint has no tokenizer: give the prompt with --prompt-ids")
+    eos = tokenizer.eos_token_id if tokenizer is not None else None
+    pages = (len(ids) + args.max_new_tokens) // 64 + 2
+    engine = engine_for(model, dtype=getattr(torch, args.dtype), page_size=64, num_pages=pages, max_batch=1, max_prefill_rows=4096)
+    try:
+        if args.sampler_temp:
+            out = sample_with_engine(engine, ids, args, eos)
+        else:
+            out = engine.generate(ids, args.max_new_tokens)
+            if eos in out:
+                out = out[:out.index(eos)]
+    finally:
+        engine.close()
+    text = tokenizer.decode(out) if (tokenizer is not None and args.prompt_ids is None) else " ".join(str(t) for t in out)
     print(text)
     return text
 

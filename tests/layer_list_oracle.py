@@ -1,0 +1,194 @@
+"""Plain float64 numpy restatement of the layer-list mechanisms, one function per mechanism, token by token where the
+mechanism is a recurrence.  Shares nothing with the product: it works on a dict of named arrays and a plain config dict of the
+Fonapel checkpoint format, and always processes a whole sequence from position 0.  Test infrastructure only.
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+
+def rms_norm(x, weight, eps, offset=0.0):
+    """x / sqrt(mean x^2 + eps) * (offset + weight) over the last axis (weight None: no weight)."""
+    y = x / np.sqrt(np.mean(x * x, axis=-1, keepdims=True) + eps)
+    return y if weight is None else y * (offset + weight)
+
+
+def rotate_pairs(z, positions, dims, base):
+    """z [L, heads, dim]: dimensions (2i, 2i+1), i < dims/2, turn by positions * base^(-2i/dims); the rest pass."""
+    out = z.copy()
+    for i in range(dims // 2):
+        ang = positions * base ** (-2.0 * i / dims)
+        c, s = np.cos(ang)[:, None], np.sin(ang)[:, None]
+        u, v = z[..., 2 * i], z[..., 2 * i + 1]
+        out[..., 2 * i] = u * c - v * s
+        out[..., 2 * i + 1] = v * c + u * s
+    return out
+
+
+def sink_attention(q, k, v, scale, sink=True):
+    """q [L, H, D], k [L, G, D], v [L, G, V]; causal; weights exp(s) / (sink + sum exp(s)).  Row by row, key by key."""
+    L, H, _ = q.shape
+    G = k.shape[1]
+    out = np.zeros((L, H, v.shape[2]))
+    for h in range(H):
+        g = h // (H // G)
+        for i in range(L):
+            s = (k[: i + 1, g] @ q[i, h]) * scale
+            e = np.exp(s)
+            out[i, h] = (e / ((1.0 if sink else 0.0) + e.sum())) @ v[: i + 1, g]
+    return out
+
+
+def short_conv_silu(z, w):
+    """z [L, C], w [C, taps] (last column multiplies the current token); zeros before the start; then SiLU."""
+    L, C = z.shape
+    taps = w.shape[1]
+    out = np.zeros_like(z)
+    for t in range(L):
+        for j in range(taps):
+            src = t - (taps - 1) + j
+            if src >= 0:
+                out[t] += w[:, j] * z[src]
+    return out / (1.0 + np.exp(-out))
+
+
+def gated_delta_rule(q, k, v, beta, g):
+    """q, k [L, G, D] (already unit / scaled), v [L, H, V], beta, g [L, H].  Per head, token by token:
+    S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q."""
+    L, H, V = v.shape
+    G, D = q.shape[1], q.shape[2]
+    out = np.zeros((L, H, V))
+    for h in range(H):
+        kh = h // (H // G)
+        S = np.zeros((D, V))
+        for t in range(L):
+            S = g[t, h] * S
+            u = beta[t, h] * (v[t, h] - S.T @ k[t, kh])
+            S = S + np.outer(k[t, kh], u)
+            out[t, h] = S.T @ q[t, kh]
+    return out
+
+
+def gelu_erf(z):
+    return 0.5 * z * (1.0 + np.vectorize(math.erf)(z / math.sqrt(2.0)))
+
+
+def sigmoid(z):
+    return 1.0 / (1.0 + np.exp(-z))
+
+
+def silu(z):
+    return z * sigmoid(z)
+
+
+def softplus(z):
+    return np.log1p(np.exp(-np.abs(z))) + np.maximum(z, 0.0)
+
+
+def layer_runs(config):
+    n = len(config["layers"])
+    loop = config.get("loop")
+    if not loop:
+        return [(i, None) for i in range(n)]
+    runs = [(i, None) for i in range(loop["start"])]
+    for t in range(loop["times"]):
+        runs += [(i, t) for i in range(loop["start"], loop["stop"])]
+    return runs + [(i, None) for i in range(loop["stop"], n)]
+
+
+def fonapel_forward(config, W, tokens, streams=None):
+    """Logits [L, vocab] of a whole sequence; ``streams`` (a list) receives the residual stream after every layer run."""
+    W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
+    eps, m = config["norm"]["eps"], config["residual_mult"]
+    L = len(tokens)
+    pos = np.arange(L, dtype=np.float64)
+    x0 = W["embed"][np.asarray(tokens)]
+    x = x0
+    for i, t in layer_runs(config):
+        spec, p = config["layers"][i], f"l{i}."
+        mc = spec["mixer"]
+        if t is not None and i == config["loop"]["start"]:
+            x = np.concatenate([x, x0], -1) @ W["loop.in"].T + W["loop.step"][t]
+        h = rms_norm(x, W[p + "norm1"], eps, offset=1.0)
+        H, G, D, V = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        if spec["type"] == "attention":
+            q = (h @ W[p + "mix.q"].T).reshape(L, H, D)
+            k = (h @ W[p + "mix.k"].T).reshape(L, G, D)
+            v = (h @ W[p + "mix.v"].T).reshape(L, G, V)
+            rot = mc.get("rot") or {"dims": 0, "base": 1.0}
+            q = rms_norm(rotate_pairs(q, pos, rot["dims"], rot["base"]), None, eps)
+            k = rms_norm(rotate_pairs(k, pos, rot["dims"], rot["base"]), None, eps)
+            o = sink_attention(q, k, v, mc["scale"]).reshape(L, H * V) * sigmoid(h @ W[p + "mix.g"].T)
+        else:
+            q = short_conv_silu(h @ W[p + "mix.q"].T, W[p + "mix.q.conv"]).reshape(L, G, D)
+            k = short_conv_silu(h @ W[p + "mix.k"].T, W[p + "mix.k.conv"]).reshape(L, G, D)
+            v = short_conv_silu(h @ W[p + "mix.v"].T, W[p + "mix.v.conv"]).reshape(L, H, V)
+            q = q / np.sqrt((q * q).sum(-1, keepdims=True) + 1e-6) * D ** -0.5
+            k = k / np.sqrt((k * k).sum(-1, keepdims=True) + 1e-6)
+            beta = sigmoid(h @ W[p + "mix.b"].T)
+            g = np.exp(-np.exp(W[p + "mix.A_log"]) * softplus(h @ W[p + "mix.a"].T + W[p + "mix.dt_bias"]))
+            o = rms_norm(gated_delta_rule(q, k, v, beta, g), W[p + "mix.norm"], eps)
+            o = o.reshape(L, H * V) * silu(h @ W[p + "mix.g"].T)
+        y = o @ W[p + "mix.o"].T
+        if spec.get("mlp"):
+            y = y + gelu_erf(h @ W[p + "mlp.up"].T) @ W[p + "mlp.down"].T
+        x = x + m * y
+        if streams is not None:
+            streams.append(x.copy())
+    return rms_norm(x, W["final.norm"], eps, offset=1.0) @ W["head"].T
+
+
+def make_fonapel_weights(config, seed=0, sigma=None):
+    """Random bf16-representable weights by tensor name (float32 arrays) for a Fonapel config dict."""
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    Wd, out = config["width"], {}
+
+    def mat(rows, cols, scale=None):
+        s = scale if scale is not None else (sigma if sigma is not None else cols ** -0.5)
+        return (torch.randn(rows, cols, generator=gen) * s).to(torch.bfloat16).float().numpy()
+
+    def vec(n, scale=0.1, shift=0.0):
+        return (torch.randn(n, generator=gen) * scale + shift).to(torch.bfloat16).float().numpy()
+
+    out["embed"], out["head"], out["final.norm"] = mat(config["vocab"], Wd, 1.0), mat(config["vocab"], Wd), vec(Wd)
+    if config.get("loop"):
+        out["loop.in"], out["loop.step"] = mat(Wd, 2 * Wd), mat(config["loop"]["times"], Wd, 0.1)
+    for i, spec in enumerate(config["layers"]):
+        p, mc = f"l{i}.", spec["mixer"]
+        H, G, D, V = mc["heads"], mc["kv_heads"], mc["dim"], mc["vdim"]
+        out[p + "norm1"] = vec(Wd)
+        if spec["type"] == "attention":
+            out[p + "mix.q"], out[p + "mix.k"], out[p + "mix.v"] = mat(H * D, Wd), mat(G * D, Wd), mat(G * V, Wd)
+        else:
+            out[p + "mix.q"], out[p + "mix.k"], out[p + "mix.v"] = mat(G * D, Wd), mat(G * D, Wd), mat(H * V, Wd)
+            for n, c in (("q", G * D), ("k", G * D), ("v", H * V)):
+                out[p + f"mix.{n}.conv"] = mat(c, mc["conv"], 0.5)
+            out[p + "mix.a"], out[p + "mix.b"] = mat(H, Wd), mat(H, Wd)
+            out[p + "mix.A_log"], out[p + "mix.dt_bias"], out[p + "mix.norm"] = vec(H, 0.5), vec(H, 0.5), vec(V, 0.1, 1.0)
+        out[p + "mix.g"], out[p + "mix.o"] = mat(H * V, Wd), mat(Wd, H * V)
+        if spec.get("mlp"):
+            out[p + "mlp.up"], out[p + "mlp.down"] = mat(spec["mlp"]["ff"], Wd), mat(Wd, spec["mlp"]["ff"])
+    return out
+
+
+def attention_layer(heads=4, kv_heads=2, dim=32, vdim=16, rot_dims=8, base=10000.0, scale=None, ff=64):
+    return {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                                           "rot": {"dims": rot_dims, "base": base}, "scale": scale if scale is not None else dim ** -0.5},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def delta_layer(heads=4, kv_heads=2, dim=16, vdim=24, conv=3, ff=64):
+    return {"type": "delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def fonapel_config(layers, width=64, vocab=101, loop=None, eps=1e-5, residual_mult=0.5):
+    cfg = {"architecture": "Fonapel", "layers": layers, "norm": {"eps": eps}, "residual_mult": residual_mult, "vocab": vocab, "width": width}
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg

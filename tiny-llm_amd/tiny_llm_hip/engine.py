@@ -304,7 +304,7 @@ _DECODE_ROW_BUCKETS = (1, 2, 3, 4, 8, 16, 32, 48, 64, 96, 128, 192, 256)
 
 def batch_generate_ids(engine: DecodeEngine, prompts: Sequence[Sequence[int]], max_new_tokens: int | Sequence[int],
                        batch_size: int, prefill_step: int = 128, eos_token_id: int | None = None,
-                       on_step=None) -> list[tuple[int, list[int]]]:
+                       on_step=None, mixed_steps: bool | None = None) -> list[tuple[int, list[int]]]:
     """Continuous batching over engine slots with the reference scheduler's shape (batch_generate,
     src/tiny_llm_ref/batch.py:136-285; benches/bench.py:run_batch_requests_serving 351-572): every loop turn
     (a) admits one pending request and prefills ONE chunk of at most ``prefill_step`` tokens in the staging slot,
@@ -312,9 +312,13 @@ def batch_generate_ids(engine: DecodeEngine, prompts: Sequence[Sequence[int]], m
     the occupied prefix of the slots (the reference steps all ``batch_size`` rows; idle rows carry context 0 and produce
     nothing, so skipping the idle tail changes no result), (d) retires finished requests and returns their pages.
     Token-id in, token-id out (no tokenizer can be downloaded here).  Needs ``engine.max_batch >= batch_size + 1``:
-    the last slot is the prefill staging slot.  Returns [(prompt_idx, generated ids)] in completion order."""
+    the last slot is the prefill staging slot.  Returns [(prompt_idx, generated ids)] in completion order.
+    ``engine``: a DecodeEngine or any engine with its request-level surface (hybrid_engine.HybridEngine).  ``mixed_steps`` (default:
+    what the engine supports): (a) and (c) of a turn run as one packed step, the prompt portion beside the decoding slots' tokens."""
     if batch_size <= 0 or prefill_step <= 0:
         raise ValueError("batch_size and prefill_step must be positive")
+    if mixed_steps is None:
+        mixed_steps = bool(getattr(engine, "supports_mixed_steps", False))
     if engine.max_batch < batch_size + 1:
         raise ValueError("engine needs batch_size + 1 slots (one prefill staging slot)")
     limits = [max_new_tokens] * len(prompts) if isinstance(max_new_tokens, int) else list(max_new_tokens)
@@ -331,15 +335,28 @@ def batch_generate_ids(engine: DecodeEngine, prompts: Sequence[Sequence[int]], m
                 engine.begin(staging)
                 live_slots.add(staging)
                 pending = {"idx": idx, "tokens": [int(t) for t in prompts[idx]], "offset": 0, "out": [], "limit": limits[idx]}
+            decoded_with_prefill: dict[int, int] | None = None
             if pending is not None:
                 total = len(pending["tokens"])
                 if pending["offset"] < total:
                     chunk = pending["tokens"][pending["offset"]:pending["offset"] + prefill_step]
                     last = pending["offset"] + len(chunk) >= total
-                    engine.prefill(staging, chunk, chunk=len(chunk), want_logits=last)
-                    pending["offset"] += len(chunk)
-                    if last:
-                        pending["out"].append(engine.read_tokens(staging, 1)[0])
+                    busy = [i for i, s in enumerate(slots) if s is not None]
+                    if mixed_steps and busy:
+                        # an engine with a packed step runs the prompt portion and the decoding slots' single tokens as ONE batch of
+                        # rows: the projections see all rows at once; each decoding slot feeds the id it generated last
+                        entries = [(staging, chunk, [len(chunk) - 1] if last else [])]
+                        entries += [(i, [slots[i]["out"][-1]], [0]) for i in busy]
+                        ids = engine.argmax(engine.step(entries))
+                        if last:
+                            pending["out"].append(ids[0])
+                        decoded_with_prefill = dict(zip(busy, ids[1 if last else 0:]))
+                        pending["offset"] += len(chunk)
+                    else:
+                        engine.prefill(staging, chunk, chunk=len(chunk), want_logits=last)
+                        pending["offset"] += len(chunk)
+                        if last:
+                            pending["out"].append(engine.read_tokens(staging, 1)[0])
                 if pending["offset"] >= total:
                     done = len(pending["out"]) >= pending["limit"] or pending["out"][-1] == eos_token_id
                     if done:
@@ -355,7 +372,18 @@ def batch_generate_ids(engine: DecodeEngine, prompts: Sequence[Sequence[int]], m
                             live_slots.add(free)
                             slots[free] = pending
                             pending = None
-            if any(s is not None for s in slots):
+            if decoded_with_prefill is not None:
+                if on_step is not None:
+                    on_step(len(decoded_with_prefill))
+                for i, token in decoded_with_prefill.items():
+                    req = slots[i]
+                    req["out"].append(token)
+                    if len(req["out"]) >= req["limit"] or token == eos_token_id:
+                        engine.release(i)
+                        live_slots.discard(i)
+                        finished.append((req["idx"], req["out"]))
+                        slots[i] = None
+            elif any(s is not None for s in slots):
                 # slots fill lowest-first, so rows above the highest occupied one are idle: decode only a bucket that
                 # covers the occupied prefix (the engine keeps one captured graph per row count; buckets bound their number)
                 def bucket(n):

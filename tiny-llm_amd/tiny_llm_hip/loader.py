@@ -301,10 +301,11 @@ class TokenizerWrapper:
         return self._detok
 
 
-def load(name_or_path: str, device: str = "cuda"):
-    """(model, tokenizer) like ``mlx_lm.load``; see the module docstring."""
+def load(name_or_path: str, device: str = "cuda", dtype: torch.dtype | None = None):
+    """(model, tokenizer) like ``mlx_lm.load``; see the module docstring.  A layer-list checkpoint without tokenizer files gives
+    (model, None)."""
     model_dir = resolve_model_dir(name_or_path)
-    model = load_weights(model_dir, device=device)
+    model = load_weights(model_dir, device=device, dtype=dtype)
     if getattr(model, "family", None) and not any((model_dir / f).is_file() for f in ("tokenizer.json", "tokenizer_config.json")):
         return model, None  # a layer-list checkpoint without tokenizer files: token ids in, token ids out
     from transformers import AutoTokenizer
