@@ -147,7 +147,7 @@ int tl_hybrid_get_stats(const tl_hybrid *e, tl_hybrid_stats *out);
 
 /* Kernel-level entry points on caller buffers (tests, microbenchmarks).  dtype as in the config. */
 int tl_hybrid_linear(int dtype, const void *a_dev, int lda, const void *w_dev, float *out_dev, int ldc, int M, int N, int K,
-                     int force_kernel /* 0 by shape, 1 row kernel, 2 tile kernel */, void *stream);
+                     int force_kernel /* 0 by shape, 1 row kernel, 2 64-wide tile kernel, 3 256-wide tile GEMM (bfloat16) */, void *stream);
 
 #ifdef __cplusplus
 }

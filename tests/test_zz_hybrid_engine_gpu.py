@@ -252,6 +252,52 @@ def test_far_keys_and_page_borders(needle_at, query):
         engine.close()
 
 
+@pytest.mark.parametrize("needle_at", [5, 255, 256, 511, 512, 640, 767, 768])
+def test_decoding_over_a_split_key_range(needle_at):
+    """From 512 keys on a single-token step splits a row's keys over workgroups (256 keys each) and merges the partial sums: the needle
+    sits at the splits' borders; the query is decoded alone, then greedy decoding goes on through the captured step."""
+    config, W, A, B = _needle_model()
+    toks = tokens_for(config, 800, seed=23, avoid=(A, B))
+    toks[needle_at] = A
+    toks[-1] = B
+    ref = O.fonapel_forward(config, W, toks)
+    engine = make_engine(config, W, page_size=16, num_pages=64, max_batch=2, max_prefill_rows=1024)
+    try:
+        engine.begin(1)
+        engine.step([(1, toks[:-1], [])])
+        n = engine.step([(1, toks[-1:], [0])])
+        assert rel_err(engine.logits_host(n), ref[-1][None]) < TOL[torch.float32]
+        engine.release(1)
+        engine.begin(0)
+        engine.prefill(0, toks[:790])
+        engine.set_token(0, toks[790])
+        engine.decode_free_running(9, [0])       # feeds 790, then its own greedy ids
+        engine.synchronize()
+        assert engine.context_len(0) == 799
+        engine.release(0)
+    finally:
+        engine.close()
+
+
+WIDE = O.fonapel_config([O.delta_layer(heads=4, kv_heads=2, dim=32, vdim=32, conv=4, ff=256), O.attention_layer(heads=4, kv_heads=2, dim=64, vdim=32, rot_dims=32, ff=256)],
+                        width=128, vocab=200, loop=(0, 2, 2))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_large_chunks_take_the_wide_tile_products(dtype):
+    """From 192 rows the bfloat16 products run on the 256-wide LDS-DMA tile GEMM with float32 epilogues; the same prompt in small
+    portions (64-wide tiles, row kernel) must give the same logits."""
+    W = O.make_fonapel_weights(WIDE, seed=24)
+    toks = tokens_for(WIDE, 300, seed=25)
+    want = O.fonapel_forward(WIDE, W, toks)
+    engine = make_engine(WIDE, W, dtype, page_size=64, num_pages=8, max_batch=2)
+    try:
+        assert rel_err(whole(engine, toks), want) < TOL[dtype]
+        assert rel_err(in_portions(engine, toks, [250, 3, 40, 1]), want) < TOL[dtype]
+    finally:
+        engine.close()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_first_tokens_where_the_sink_weighs_most(dtype):
     """At position 0 a weight is exp(s) / (1 + exp(s)): without the 1 in the denominator it would be exactly 1."""
@@ -365,8 +411,9 @@ def test_checkpoint_directory_through_loader_registry_and_command_line(tmp_path,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(1, 64, 128), (3, 50, 77), (8, 300, 256), (9, 64, 64), (70, 130, 96), (200, 97, 203), (64, 64, 8)])
-@pytest.mark.parametrize("kernel", [0, 1, 2])
+@pytest.mark.parametrize("shape", [(1, 64, 128), (3, 50, 77), (8, 300, 256), (9, 64, 64), (70, 130, 96), (200, 97, 203), (64, 64, 8), (256, 512, 256),
+                                   (300, 132, 128), (1000, 260, 192)])
+@pytest.mark.parametrize("kernel", [0, 1, 2, 3])
 def test_linear_kernels_against_torch(shape, dtype, kernel):
     import ctypes
 
@@ -375,6 +422,8 @@ def test_linear_kernels_against_torch(shape, dtype, kernel):
     M, N, K = shape
     if kernel == 1 and M > 8:
         pytest.skip("the row kernel takes at most 8 rows")
+    if kernel == 3 and (dtype != torch.bfloat16 or K % 64 or K < 128 or N % 4):
+        pytest.skip("the 256-wide tile GEMM takes bfloat16, whole 64-wide K steps (two at least) and columns in fours")
     gen = torch.Generator().manual_seed(M * 1000 + N)
     a = torch.randn(M, K, generator=gen).to(dtype).cuda()
     w = torch.randn(N, K, generator=gen).to(dtype).cuda()

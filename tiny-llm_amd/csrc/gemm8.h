@@ -30,7 +30,11 @@ struct Gemm8Args {
     uint16_t *out;             // [M, N]  (EPI_SWIGLU: [M, N / 2], weight rows interleaved gate_i, up_i)
     const uint16_t *residual;  // EPI_RESIDUAL [M, N]
     int M, N, K;
+    float *out_f32 = nullptr;  // EPI_F32_STORE / EPI_F32_AXPY: [M, N] float32 (a float32 residual stream or float32 projections behind bf16 operands)
+    float alpha = 1.f;         // EPI_F32_AXPY: out_f32 += alpha * product
 };
+// epilogues beside EPI_STORE / EPI_RESIDUAL / EPI_SWIGLU (qmv.h): the accumulators leave as float32
+enum { EPI_F32_STORE = 3, EPI_F32_AXPY = 4 };
 
 constexpr int G8_BK = 64, G8_WAVES = 8;
 #ifdef G8_TRACE  // tools/lab/gemm8_lab only: wall-clock stamps of wave 0 of workgroup G8_TRACE behind every step's barrier (and around a tile's epilogue)

@@ -82,9 +82,13 @@ static int launch8_tile(const Gemm8Args &a, const Gemm8Plan &pl, hipStream_t st)
 }
 
 int launch_gemm8_bf16(const Gemm8Args &args, int epi, hipStream_t st) {
-    if (!args.a || !args.w || !args.out) return -1;
+    const bool f32_out = epi == EPI_F32_STORE || epi == EPI_F32_AXPY;
+    if (!args.a || !args.w || (f32_out ? !args.out_f32 : !args.out)) return -1;
     const Gemm8Plan pl = gemm8_plan(args.M, args.N, args.K);
     if (!pl.ok) return -1;
+    if (f32_out && (size_t)args.M * args.N * 4 >= (1ull << 31)) return -1;
+    if (epi == EPI_F32_STORE) return launch8_tile<EPI_F32_STORE>(args, pl, st);
+    if (epi == EPI_F32_AXPY) return launch8_tile<EPI_F32_AXPY>(args, pl, st);
     if (epi == EPI_RESIDUAL && !args.residual) return -1;
     if (epi == EPI_STORE) return launch8_tile<EPI_STORE>(args, pl, st);
     if (epi == EPI_RESIDUAL) return launch8_tile<EPI_RESIDUAL>(args, pl, st);

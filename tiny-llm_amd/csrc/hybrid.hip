@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -14,6 +15,7 @@
 
 #include "../../include/tinyllm_hybrid.h"
 #include "common.h"
+#include "gemm8.h"
 #include "hybrid_kernels.h"
 #include "page_pool.h"
 
@@ -29,6 +31,14 @@
     } while (0)
 
 namespace tl {
+int qmm3_num_cus() {  // gemm8.hip sizes its persistent grid by the CU count
+    static int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        return n;
+    }();
+    return cus;
+}
 namespace hy {
 
 struct Run {
@@ -58,6 +68,8 @@ struct tl_hybrid {
     bool table_dirty = true;
     int32_t *table_dev = nullptr;
     // workspace
+    float *part_acc = nullptr, *part_ml = nullptr;  // attention partials of split key ranges: [max_slots, heads, 64, vdim] / [..., 2]
+    bool attn_rows_only = false;                    // TL_HYBRID_ATTN_ROWS=1: the one-wave-per-row attention everywhere (A/B twin of the tile kernel)
     float *x = nullptr, *x0 = nullptr, *proj = nullptr, *qbuf = nullptr, *conv_out = nullptr, *obuf = nullptr, *logits = nullptr;
     void *h = nullptr, *cat = nullptr, *cat2 = nullptr, *hsel = nullptr;
     int ld_proj = 0, ld_cat = 0;
@@ -121,6 +133,23 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
     const int vec_ok = (K % 8 == 0) && (lda % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
     const bool rows = force == 1 || (force == 0 && M <= 8);
     TL_REQUIRE(!rows || M <= 8, "hybrid linear: the row kernel takes at most 8 rows");
+    if constexpr (sizeof(S) == 2) {
+        // large bf16 products: the framework's LDS-DMA 256-wide tile GEMM with its float32 epilogues (gemm8.h); dense operands, whole 64-wide K steps
+        const bool big = force == 3 || (force == 0 && M >= 192);
+        if (big && lda == K && ldc == N && gemm8_applicable(M, N, K) && (size_t)M * N * 4 < (1ull << 31)) {
+            Gemm8Args g{};
+            g.a = (const uint16_t *)A, g.w = (const uint16_t *)W, g.M = M, g.N = N, g.K = K, g.out_f32 = out, g.alpha = alpha;
+            if (launch_gemm8_bf16(g, epi == 1 ? EPI_F32_AXPY : EPI_F32_STORE, st) == 0) {
+                if (epi == 2) {
+                    const size_t n = (size_t)M * N;
+                    hipLaunchKernelGGL(add_rowvec_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, out, bias, N, M);
+                    TL_CHECK_LAUNCH("hybrid linear bias");
+                }
+                return TL_OK;
+            }
+        }
+        TL_REQUIRE(force != 3, "hybrid linear: the 256-wide tile GEMM does not take this shape");
+    }
     if (rows) {
         dim3 grid((N + 3) / 4), block(256);
         if (epi == 0) hipLaunchKernelGGL((gemm_rows_kernel<D, 0>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
@@ -136,7 +165,7 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
     return TL_OK;
 }
 
-static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs) {
+static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
     // lanes per state column R and rows per lane RPT: key_dim <= RPT * R; a workgroup takes VB columns with VB * R <= 256 threads
     int rpt = 8;
     while (rpt < 128 && (L.dim + rpt - 1) / rpt > 16) rpt *= 2;
@@ -151,7 +180,7 @@ static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run 
     const int C = conv_channels(L);
     const int a0 = 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim, b0 = a0 + L.heads;
 #define HY_DELTA(RPT)                                                                                                                          \
-    hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, lds, e->stream, e->conv_out, C, e->proj, e->ld_proj, a0, b0, L.a_log_dev, L.dt_bias_dev, \
+    hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, lds, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
                        L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim, R, VB, TB)
     switch (rpt) {
         case 8: HY_DELTA(8); break;
@@ -165,9 +194,54 @@ static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run 
     return TL_OK;
 }
 
-// every layer run over `rows` packed rows described by m
+struct StepShape {
+    int rows, n_seqs, max_len;         // packed rows, sequences, longest chunk
+    int n_splits = 1, keys_per_split = 1 << 30;  // attention: the key range of a row split over workgroups (decode steps over long contexts)
+};
+
+// how a step's attention splits the keys: only steps of single tokens, from 512 keys on; 256 keys per split, doubled until at most 64 splits
+static void plan_splits(StepShape &sh, int ctx_bound) {
+    sh.n_splits = 1;
+    sh.keys_per_split = 1 << 30;
+    if (sh.max_len != 1 || ctx_bound <= 512) return;
+    int kps = 256;
+    while ((ctx_bound + kps - 1) / kps > 64) kps *= 2;
+    int n = 1;
+    while (n * kps < ctx_bound) n *= 2;
+    sh.n_splits = n;
+    sh.keys_per_split = kps;
+}
+
+template <typename D, int DK4, int VT>
+static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, const StepShape &sh, const float *gate, int ldg,
+                            int ldo) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    const int HG = L.heads / L.kv_heads;
+    int HGB = 1;
+    while (HGB < HG && HGB < 16) HGB *= 2;
+    const int n_hblk = (HG + HGB - 1) / HGB, TQ = 64 / HGB;
+    const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
+    const size_t lds = (size_t)64 * ((4 * dk4 + 4) + (16 * vt_n + 4)) * 4;
+    auto kern = attn_tile_kernel<D, DK4, VT>;
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    dim3 grid((sh.max_len + TQ - 1) / TQ, L.kv_heads * n_hblk, sh.n_seqs * sh.n_splits);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)run.kpool, (const S *)run.vpool, m.seq_row0, m.seq_slot, m.row_pos,
+                       e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.sink, HGB, n_hblk, sh.keys_per_split,
+                       sh.n_splits, gate, ldg, (S *)e->cat, ldo, e->part_acc, e->part_ml);
+    TL_CHECK_LAUNCH("hybrid attention tile");
+    if (sh.n_splits > 1) {
+        hipLaunchKernelGGL((attn_merge_kernel<D>), dim3(sh.rows, L.heads), dim3(64), 0, e->stream, e->part_acc, e->part_ml, sh.n_splits, L.heads, L.vdim, gate,
+                           ldg, (S *)e->cat, ldo);
+        TL_CHECK_LAUNCH("hybrid attention merge");
+    }
+    return TL_OK;
+}
+
+// every layer run over the packed rows described by m
 template <typename D>
-static int forward_t(tl_hybrid *e, const Meta &m, int rows, int n_seqs) {
+static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
+    const int rows = sh.rows, n_seqs = sh.n_seqs;
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
     hipStream_t st = e->stream;
@@ -185,43 +259,53 @@ static int forward_t(tl_hybrid *e, const Meta &m, int rows, int n_seqs) {
         hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(256), 0, st, e->x, L.norm_dev, L.norm_offset, c.norm_eps, (S *)e->h, W, (const int32_t *)nullptr);
         TL_CHECK_LAUNCH("hybrid norm");
         const int nin = in_cols(L), HV = L.heads * L.vdim;
-        HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, e->ld_proj, rows, nin, W, 0, 1.f, nullptr, 0, st));
+        const int ldp = nin, ldcat = HV + L.ff;  // dense rows: a layer's buffers are as wide as the layer needs
+        HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, ldp, rows, nin, W, 0, 1.f, nullptr, 0, st));
         if (L.kind == TL_MIX_ATTENTION) {
             const int H = L.heads, G = L.kv_heads;
-            hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, e->ld_proj, m.row_seq, m.row_pos, m.seq_slot,
+            hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot,
                                e->table_dev, c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.qk_unit_rms, c.norm_eps, H, G, L.dim,
                                L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
             TL_CHECK_LAUNCH("hybrid attention prep");
             const float *gate = L.gated ? e->proj + (size_t)(H + G) * L.dim + (size_t)G * L.vdim : nullptr;
-            hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(rows, H), dim3(64), (L.dim + 64) * sizeof(float), st, e->qbuf, (const S *)run.kpool,
-                               (const S *)run.vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, H, G, L.dim, L.vdim,
-                               L.scale, L.sink, gate, e->ld_proj, (S *)e->cat, e->ld_cat);
-            TL_CHECK_LAUNCH("hybrid attention");
+            const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
+            if (e->attn_rows_only || dk4 > 64 || vt_n > 16) {
+                hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(rows, H), dim3(64), (L.dim + 64) * sizeof(float), st, e->qbuf, (const S *)run.kpool,
+                                   (const S *)run.vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, H, G, L.dim, L.vdim,
+                                   L.scale, L.sink, gate, ldp, (S *)e->cat, ldcat);
+                TL_CHECK_LAUNCH("hybrid attention");
+            } else if (dk4 <= 16 && vt_n <= 4) {
+                HY_TRY((launch_attn_tile<D, 16, 4>(e, L, run, m, sh, gate, ldp, ldcat)));
+            } else if (dk4 <= 32 && vt_n <= 8) {
+                HY_TRY((launch_attn_tile<D, 32, 8>(e, L, run, m, sh, gate, ldp, ldcat)));
+            } else {
+                HY_TRY((launch_attn_tile<D, 64, 16>(e, L, run, m, sh, gate, ldp, ldcat)));
+            }
         } else {
             const int C = conv_channels(L);
             const size_t n = (size_t)rows * C;
-            hipLaunchKernelGGL(conv_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, e->ld_proj, L.conv_dev, L.conv_taps, C, m.row_seq,
+            hipLaunchKernelGGL(conv_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, L.conv_dev, L.conv_taps, C, m.row_seq,
                                m.seq_row0, m.seq_slot, run.conv_state, e->conv_out, rows);
             TL_CHECK_LAUNCH("hybrid conv");
             if (L.conv_taps > 1) {
-                hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)(((size_t)n_seqs * C + 255) / 256)), dim3(256), 0, st, e->proj, e->ld_proj, L.conv_taps, C,
+                hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)(((size_t)n_seqs * C + 255) / 256)), dim3(256), 0, st, e->proj, ldp, L.conv_taps, C,
                                    m.seq_row0, m.seq_slot, run.conv_state, n_seqs);
                 TL_CHECK_LAUNCH("hybrid conv state");
             }
-            HY_TRY(launch_delta(e, L, run, m, n_seqs));
+            HY_TRY(launch_delta(e, L, run, m, n_seqs, ldp));
             const float *gate = e->proj + (size_t)C;
-            hipLaunchKernelGGL((delta_out_kernel<D>), dim3(rows, L.heads), dim3(64), 0, st, e->obuf, L.out_norm_dev, c.norm_eps, gate, e->ld_proj, L.heads,
-                               L.vdim, (S *)e->cat, e->ld_cat);
+            hipLaunchKernelGGL((delta_out_kernel<D>), dim3(rows, L.heads), dim3(64), 0, st, e->obuf, L.out_norm_dev, c.norm_eps, gate, ldp, L.heads,
+                               L.vdim, (S *)e->cat, ldcat);
             TL_CHECK_LAUNCH("hybrid delta out");
         }
         if (L.ff > 0) {
             const size_t n = (size_t)rows * L.ff;
-            hipLaunchKernelGGL((ff_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, e->ld_proj, nin - L.ff, L.ff, L.ff_act,
-                               (S *)e->cat, e->ld_cat, HV, rows);
+            hipLaunchKernelGGL((ff_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, nin - L.ff, L.ff, L.ff_act,
+                               (S *)e->cat, ldcat, HV, rows);
             TL_CHECK_LAUNCH("hybrid ff act");
         }
         // x += m * ([mixer out ; ff act] . [W_o | W_down]^T)
-        HY_TRY(linear_t<D>(e->cat, e->ld_cat, L.w_out_dev, e->x, W, rows, W, HV + L.ff, 1, c.residual_mult, nullptr, 0, st));
+        HY_TRY(linear_t<D>(e->cat, ldcat, L.w_out_dev, e->x, W, rows, W, HV + L.ff, 1, c.residual_mult, nullptr, 0, st));
         if (e->trace && e->trace_buf && rows <= c.max_rows)
             HY_HIP(hipMemcpyAsync(e->trace_buf + ri * (size_t)c.max_rows * W, e->x, (size_t)rows * W * 4, hipMemcpyDeviceToDevice, st));
     }
@@ -244,8 +328,8 @@ static int head_t(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
     return TL_OK;
 }
 
-static int forward(tl_hybrid *e, const Meta &m, int rows, int n_seqs) {
-    return e->cfg.dtype == TL_HY_BF16 ? forward_t<BF16>(e, m, rows, n_seqs) : forward_t<F32>(e, m, rows, n_seqs);
+static int forward(tl_hybrid *e, const Meta &m, const StepShape &sh) {
+    return e->cfg.dtype == TL_HY_BF16 ? forward_t<BF16>(e, m, sh) : forward_t<F32>(e, m, sh);
 }
 static int head(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
     return e->cfg.dtype == TL_HY_BF16 ? head_t<BF16>(e, m, n_want, set_pending) : head_t<F32>(e, m, n_want, set_pending);
@@ -393,6 +477,12 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     HY_TRY(dev_alloc(p, &e->conv_out, (size_t)R * std::max(1, max_c)));
     HY_TRY(dev_alloc(p, &e->obuf, (size_t)R * std::max(1, max_hv)));
     HY_TRY(dev_alloc(p, &e->logits, (size_t)R * c.vocab));
+    int max_h = 1, max_v = 1;
+    for (const tl_hybrid_layer &L : e->layers)
+        if (L.kind == TL_MIX_ATTENTION) max_h = std::max(max_h, L.heads), max_v = std::max(max_v, L.vdim);
+    HY_TRY(dev_alloc(p, &e->part_acc, (size_t)c.max_slots * max_h * 64 * max_v));
+    HY_TRY(dev_alloc(p, &e->part_ml, (size_t)c.max_slots * max_h * 64 * 2));
+    if (const char *v = getenv("TL_HYBRID_ATTN_ROWS")) e->attn_rows_only = v[0] != '\0' && v[0] != '0';
     HY_TRY(dev_alloc(p, (char **)&e->h, (size_t)R * W * es));
     HY_TRY(dev_alloc(p, (char **)&e->hsel, (size_t)R * W * es));
     HY_TRY(dev_alloc(p, (char **)&e->cat, (size_t)R * e->ld_cat * es, true));
@@ -519,7 +609,14 @@ extern "C" int tl_hybrid_step(tl_hybrid *e, int n_seqs, const int *slots, const 
     }
     HY_HIP(hipMemcpyAsync(e->meta_dev, e->meta_host, meta_ints(R, S) * 4, hipMemcpyHostToDevice, e->stream));
     HY_TRY(sync_table(e));
-    HY_TRY(forward(e, e->meta, (int)rows, n_seqs));
+    StepShape sh{(int)rows, n_seqs, 0};
+    int ctx_bound = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+        sh.max_len = std::max(sh.max_len, lens[i]);
+        ctx_bound = std::max(ctx_bound, e->pool->context(slots[i]) + lens[i]);
+    }
+    plan_splits(sh, ctx_bound);
+    HY_TRY(forward(e, e->meta, sh));
     HY_TRY(head(e, e->meta, n_want, true));
     for (int i = 0; i < n_seqs; ++i) e->pool->advance(slots[i], lens[i]);
     e->last_rows = n_want;
@@ -546,10 +643,17 @@ extern "C" int tl_hybrid_decode(tl_hybrid *e, int n_seqs, const int *slots, int 
     TL_REQUIRE(n_seqs <= c.max_rows, "hybrid_decode: more sequences than max_rows");
     std::vector<int> extra(n_seqs, steps);
     HY_TRY(reserve_all(e, n_seqs, slots, extra.data()));
-    const std::vector<int> key(slots, slots + n_seqs);
+    StepShape sh{n_seqs, n_seqs, 1};
+    int ctx_bound = 0;
+    for (int i = 0; i < n_seqs; ++i) ctx_bound = std::max(ctx_bound, e->pool->context(slots[i]) + steps);
+    plan_splits(sh, ctx_bound);
+    const std::vector<int> slot_list(slots, slots + n_seqs);
+    std::vector<int> key(slot_list);  // a captured step holds its slots and its split of the key range
+    key.push_back(sh.n_splits);
+    key.push_back(sh.keys_per_split);
     HY_HIP(hipStreamSynchronize(e->stream));
     const int R = c.max_rows, S = c.max_slots;
-    if (e->dmeta_slots != key) {  // static part of the decode metadata: row i <-> sequence i <-> slots[i]
+    if (e->dmeta_slots != slot_list) {  // static part of the decode metadata: row i <-> sequence i <-> slots[i]
         Meta hm = carve(e->meta_host, R, S);
         std::memset(e->meta_host, 0, meta_ints(R, S) * 4);
         for (int i = 0; i < n_seqs; ++i) {
@@ -562,7 +666,7 @@ extern "C" int tl_hybrid_decode(tl_hybrid *e, int n_seqs, const int *slots, int 
         hm.seq_row0[n_seqs] = n_seqs;
         HY_HIP(hipMemcpyAsync(e->dmeta_dev, e->meta_host, meta_ints(R, S) * 4, hipMemcpyHostToDevice, e->stream));
         HY_HIP(hipStreamSynchronize(e->stream));
-        e->dmeta_slots = key;
+        e->dmeta_slots = slot_list;
     }
     std::vector<int32_t> ctx(S, 0);
     for (int s = 0; s < S; ++s) ctx[s] = e->pool->live(s) ? e->pool->context(s) : 0;
@@ -573,7 +677,7 @@ extern "C" int tl_hybrid_decode(tl_hybrid *e, int n_seqs, const int *slots, int 
         hipLaunchKernelGGL(decode_meta_kernel, dim3((n_seqs + 63) / 64), dim3(64), 0, e->stream, e->dmeta.seq_slot, n_seqs, e->pending_dev, e->ctx_dev,
                            e->dmeta.tokens, e->dmeta.row_pos, 0);
         TL_CHECK_LAUNCH("hybrid decode meta");
-        HY_TRY(forward(e, e->dmeta, n_seqs, n_seqs));
+        HY_TRY(forward(e, e->dmeta, sh));
         HY_TRY(head(e, e->dmeta, n_seqs, true));
         hipLaunchKernelGGL(decode_meta_kernel, dim3((n_seqs + 63) / 64), dim3(64), 0, e->stream, e->dmeta.seq_slot, n_seqs, e->pending_dev, e->ctx_dev,
                            e->dmeta.tokens, e->dmeta.row_pos, 1);

@@ -368,6 +368,182 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
     }
 }
 
+// ---- attention, step 2 (tile form): float32 MFMA flash attention over the paged K/V, grouped heads sharing the staged tiles -----------
+// A workgroup (4 waves) owns 64 "query rows" of one sequence and one K/V head: row rho = (token rho / HGB, head-in-group rho % HGB), HGB = the
+// group's query heads rounded up to a power of two (<= 16; larger groups take several workgroups), so K and V tiles are staged once for
+// every query head that reads them.  Keys come in tiles of 64, converted to float32 in LDS; both products run on v_mfma_f32_16x16x4_f32
+// (full float32 products), transposed so that no value crosses lanes between them:
+//   S^T[key, row]  = K . Q^T      A = K tile (LDS), B = this wave's 16 query rows (registers, scale folded in)
+//   O^T[vcol, row] = V^T . P^T    A = V tile (LDS), B = the weights exactly where the first product left them: the k-slot of lane group g in
+//                                 step r is key 4 g + r of the 16-key sub-tile (a sum does not care in which order its terms are paired)
+// Per query row (= per lane column) a running maximum and sum; the sink is their start value (0, 1).  The key range may be split over
+// gridDim.z (decode steps over long contexts): then unnormalised partial sums + (max, sum) go to part_* and attn_merge_kernel finishes.
+template <typename D, int DK4, int VT>
+__global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
+                                                        const int32_t *seq_row0, const int32_t *seq_slot, const int32_t *row_pos,
+                                                        const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
+                                                        float scale, int sink, int HGB, int n_hblk, int keys_per_split, int n_splits, const float *gate,
+                                                        int ldg, typename D::storage *out, int ldo, float *part_acc, float *part_ml) {
+    using S = typename D::storage;
+    extern __shared__ float smem[];
+    const int dk4 = (dim + 3) / 4, DKP = 4 * dk4 + 4, vt_n = (vdim + 15) / 16, VP = 16 * vt_n + 4;
+    float *Ks = smem;             // [64][DKP]
+    float *Vs = smem + 64 * DKP;  // [64][VP]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, col = lane & 15;
+    const int seq = blockIdx.z / n_splits, split = blockIdx.z % n_splits;
+    const int kvh = blockIdx.y / n_hblk, hblk = blockIdx.y % n_hblk, HG = H / G, TQ = 64 / HGB;
+    const int r0 = seq_row0[seq], len = seq_row0[seq + 1] - r0, t0 = blockIdx.x * TQ;
+    if (t0 >= len) return;
+    const int pos0 = row_pos[r0], slot = seq_slot[seq];
+    const int32_t *bt = block_table + (size_t)slot * max_pages;
+    const int k_end_tile = pos0 + min(t0 + TQ, len);  // keys the tile's last query row sees
+    const int k_begin = split * keys_per_split, k_end = min(k_end_tile, (split + 1) * keys_per_split);
+    // this lane's query row (column of the transposed products)
+    const int rho = wave * 16 + col, tl = rho / HGB, hb = hblk * HGB + rho % HGB;
+    const bool row_ok = t0 + tl < len && hb < HG;
+    const int trow = r0 + t0 + tl, head = kvh * HG + hb, qpos = pos0 + t0 + tl;
+    float m_run = (sink && split == 0) ? 0.f : -INFINITY, l_run = (sink && split == 0) ? 1.f : 0.f;
+    f32x4 o[VT];
+#pragma unroll
+    for (int v = 0; v < VT; ++v) o[v] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k_begin < k_end) {
+        float qf[DK4];
+#pragma unroll
+        for (int kk = 0; kk < DK4; ++kk) {
+            const int d = 4 * kk + g4;
+            qf[kk] = (row_ok && d < dim) ? qbuf[((size_t)trow * H + head) * dim + d] * scale : 0.f;
+        }
+        for (int kb = k_begin; kb < k_end; kb += 64) {
+            __syncthreads();
+            for (int i = tid; i < 64 * dk4; i += 256) {  // K tile -> float32
+                const int key = i / dk4, c4 = i % dk4, j = kb + key;
+                f32x4 v{0.f, 0.f, 0.f, 0.f};
+                if (j < k_end) {
+                    const S *src = kpool + (((size_t)bt[j / page_size] * G + kvh) * page_size + j % page_size) * dim + 4 * c4;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (4 * c4 + e < dim) v[e] = D::to_float(src[e]);
+                }
+                *reinterpret_cast<f32x4 *>(Ks + key * DKP + 4 * c4) = v;
+            }
+            const int v4 = 4 * vt_n;
+            for (int i = tid; i < 64 * v4; i += 256) {  // V tile -> float32
+                const int key = i / v4, c4 = i % v4, j = kb + key;
+                f32x4 v{0.f, 0.f, 0.f, 0.f};
+                if (j < k_end) {
+                    const S *src = vpool + (((size_t)bt[j / page_size] * G + kvh) * page_size + j % page_size) * vdim + 4 * c4;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (4 * c4 + e < vdim) v[e] = D::to_float(src[e]);
+                }
+                *reinterpret_cast<f32x4 *>(Vs + key * VP + 4 * c4) = v;
+            }
+            __syncthreads();
+            f32x4 sc[4];
+            float m_tile = -INFINITY;
+#pragma unroll
+            for (int n = 0; n < 4; ++n) {
+                f32x4 a4{0.f, 0.f, 0.f, 0.f};
+                const float *kr = Ks + (16 * n + col) * DKP + g4;
+#pragma unroll
+                for (int kk = 0; kk < DK4; ++kk)
+                    if (kk < dk4) a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk], qf[kk], a4, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = kb + 16 * n + 4 * g4 + r;
+                    a4[r] = (row_ok && j <= qpos && j < k_end) ? a4[r] : -INFINITY;
+                    m_tile = fmaxf(m_tile, a4[r]);
+                }
+                sc[n] = a4;
+            }
+            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
+            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+            const float m_new = fmaxf(m_run, m_tile);
+            const float corr = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);
+            float psum = 0.f;
+#pragma unroll
+            for (int n = 0; n < 4; ++n)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float p = (sc[n][r] == -INFINITY) ? 0.f : expf(sc[n][r] - m_new);
+                    sc[n][r] = p;
+                    psum += p;
+                }
+            psum += __shfl_xor(psum, 16, 64);
+            psum += __shfl_xor(psum, 32, 64);
+            l_run = l_run * corr + psum;
+            m_run = m_new;
+#pragma unroll
+            for (int v = 0; v < VT; ++v)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[v][r] *= corr;
+#pragma unroll
+            for (int n = 0; n < 4; ++n)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float *vr = Vs + (16 * n + 4 * g4 + r) * VP + col;
+#pragma unroll
+                    for (int v = 0; v < VT; ++v)
+                        if (v < vt_n) o[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[n][r], o[v], 0, 0, 0);
+                }
+        }
+    }
+    if (!row_ok) return;
+    if (n_splits == 1) {
+        const float invl = l_run > 0.f ? 1.f / l_run : 0.f;
+#pragma unroll
+        for (int v = 0; v < VT; ++v)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int c = 16 * v + 4 * g4 + r;
+                if (v < vt_n && c < vdim) {
+                    float val = o[v][r] * invl;
+                    if (gate) val *= sigmoid_f(gate[(size_t)trow * ldg + (size_t)head * vdim + c]);
+                    out[(size_t)trow * ldo + (size_t)head * vdim + c] = D::from_float(val);
+                }
+            }
+    } else {
+        const size_t pi = ((size_t)trow * H + head) * n_splits + split;
+#pragma unroll
+        for (int v = 0; v < VT; ++v)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int c = 16 * v + 4 * g4 + r;
+                if (v < vt_n && c < vdim) part_acc[pi * vdim + c] = o[v][r];
+            }
+        if (g4 == 0) {
+            part_ml[2 * pi] = m_run;
+            part_ml[2 * pi + 1] = l_run;
+        }
+    }
+}
+
+// the splits of a row's key range put together: one wave per (row, query head)
+template <typename D>
+__global__ __launch_bounds__(64) void attn_merge_kernel(const float *part_acc, const float *part_ml, int n_splits, int H, int vdim, const float *gate,
+                                                        int ldg, typename D::storage *out, int ldo) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const size_t p0 = ((size_t)t * H + h) * n_splits;
+    float M = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[2 * (p0 + s)]);
+    float L = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float m = part_ml[2 * (p0 + s)];
+        if (m != -INFINITY) L += part_ml[2 * (p0 + s) + 1] * expf(m - M);
+    }
+    const float invl = L > 0.f ? 1.f / L : 0.f;
+    for (int c = lane; c < vdim; c += 64) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float m = part_ml[2 * (p0 + s)];
+            if (m != -INFINITY) acc += part_acc[(p0 + s) * vdim + c] * expf(m - M);
+        }
+        float val = acc * invl;
+        if (gate) val *= sigmoid_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]);
+        out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(val);
+    }
+}
+
 // ---- feed-forward activation: cat[t, col0 + c] = act(proj[t, up0 + c]) ---------------------------------------------------
 template <typename D>
 __global__ void ff_act_kernel(const float *proj, int ldp, int up0, int ff, int kind, typename D::storage *out, int ldo, int col0, int rows) {

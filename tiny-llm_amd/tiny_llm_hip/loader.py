@@ -118,9 +118,11 @@ def load_weights(model_dir: str | Path, device: str = "cuda", dtype: torch.dtype
     torch.float32, the precision the engine will run in)."""
     model_dir = Path(model_dir)
     config = json.loads((model_dir / "config.json").read_text())
-    from .layer_list import FAMILIES
+    if "architecture" in config:  # a layer-list family names itself (MLX checkpoints carry "model_type" / "architectures")
+        from .layer_list import FAMILIES
 
-    if config.get("architecture") in FAMILIES:
+        if config["architecture"] not in FAMILIES:
+            raise ValueError(f"unknown architecture {config['architecture']!r}: layer-list families are {sorted(FAMILIES)}")
         return _load_layer_list(model_dir, config, dtype)
     if dtype not in (None, torch.bfloat16):
         raise ValueError("the W4A16 path runs in bfloat16 only")
