@@ -842,7 +842,15 @@ def main() -> None:
                          "frac from its kernel durations; committed: replay the newest committed summary; off: in-kernel stamps only")
     ap.add_argument("--engine", default="hip", choices=("hip", "sleep"),
                     help="sleep = launch-path plumbing test without a GPU (gloo); never a measurement")
+    ap.add_argument("--layer-list", default=None, metavar="WIDTHS",
+                    help="instead of the default workload: prefill / decode throughput of a layer-list model (Fonapel family) beside Qwen3 W4A16 at "
+                         "equal layer sizes, e.g. 1024,2048,4096 (benches/layer_list_compare.py; one JSON line of its own, --prompt-len / --steps apply)")
     args = ap.parse_args()
+    if args.layer_list is not None:
+        from benches import layer_list_compare
+
+        layer_list_compare.main([int(w) for w in args.layer_list.split(",") if w], args.prompt_len or 2048, args.steps or 64)
+        return
     t_start = time.perf_counter()
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         self_launch(sys.argv[1:], args.gpus)  # does not return

@@ -1,0 +1,166 @@
+"""Throughput of a layer-list model (the Fonapel family on the layer-list engine) beside the framework's closest existing
+model, Qwen3 on the fused W4A16 engine, at equal layer sizes and with random weights:  `python bench.py --layer-list W[,W...]`.
+
+Per width W (head width 128, W/128 query heads, a quarter of them K/V heads, feed-forward 3 W, 4 layers, vocabulary 32,768):
+prefill of one prompt in one chunk, decode of 1 and of 4 sequences over that context.  Beside tokens/s every leg reports what
+its roofline is made of -- the bytes a decode step must stream (weights once + K/V or state of every live sequence), the
+multiply-adds of a prefill chunk -- and the fraction of 8 TB/s / 2.5 PFLOP/s (dense bf16) that the measured time amounts to.
+The two models differ where the designs differ: bf16 matrices against 4-bit ones (4 x the bytes per decode step), two of
+four mixers recurrent (no K/V to stream, a sequential recurrence in prefill), one fused in/out product pair per layer.
+"""
+
+from __future__ import annotations
+
+import json
+import random
+import time
+
+HBM_BYTES_PER_S = 8.0e12
+BF16_FLOPS = 2.5e15
+
+
+def fonapel_config(width: int, layers: int = 4, vocab: int = 32768) -> dict:
+    heads = max(1, width // 128)
+    kv = max(1, heads // 4)
+    attn = {"type": "attention", "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "rot": {"dims": 64, "base": 1e6}, "scale": 128 ** -0.5},
+            "mlp": {"kind": "dense", "ff": 3 * width}}
+    delta = {"type": "delta", "mixer": {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4}, "mlp": {"kind": "dense", "ff": 3 * width}}
+    order = [delta, attn, attn, delta]
+    return {"architecture": "Fonapel", "layers": [order[i % 4] for i in range(layers)], "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": vocab,
+            "width": width}
+
+
+def qwen3_config(width: int, layers: int = 4, vocab: int = 32768) -> dict:
+    heads = max(1, width // 128)
+    return dict(hidden_size=width, num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=max(1, heads // 4), head_dim=128,
+                intermediate_size=3 * width, vocab_size=vocab, rope_theta=1000000, rms_norm_eps=1e-6, max_position_embeddings=40960,
+                tie_word_embeddings=False)
+
+
+def fonapel_costs(cfg: dict, ctx: int, dtype_bytes: int = 2) -> dict:
+    """Matrix elements (= multiply-adds per token), attention multiply-adds of a causal prompt, and the bytes a decode step streams."""
+    W, params, kv_per_tok, state = cfg["width"], 0, 0, 0
+    for L in cfg["layers"]:
+        m, ff = L["mixer"], (L["mlp"] or {}).get("ff", 0)
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        if L["type"] == "attention":
+            params += W * (H * D + G * D + G * V + H * V) + H * V * W
+            kv_per_tok += G * (D + V)
+        else:
+            params += W * (2 * G * D + 2 * H * V + 2 * H) + H * V * W
+            state += H * D * V
+        params += 2 * W * ff
+    attn_macs = sum(L["mixer"]["heads"] * (L["mixer"]["dim"] + L["mixer"]["vdim"]) for L in cfg["layers"] if L["type"] == "attention")
+    head = cfg["vocab"] * W
+    return {"matrix_elems": params, "head_elems": head, "attn_macs_per_pair": attn_macs,
+            "decode_bytes": lambda b: (params + head) * dtype_bytes + b * (ctx * kv_per_tok * dtype_bytes + 2 * state * 4)}
+
+
+def qwen3_costs(cfg: dict, ctx: int) -> dict:
+    W, H, G, D, I = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["intermediate_size"]
+    per_layer = W * (H * D + 2 * G * D) + H * D * W + 3 * W * I
+    params = per_layer * cfg["num_hidden_layers"]
+    head = cfg["vocab_size"] * W
+    w4 = 0.5 + 4.0 / 128  # nibbles + bf16 scale and bias per group of 128
+    return {"matrix_elems": params, "head_elems": head, "attn_macs_per_pair": cfg["num_hidden_layers"] * H * 2 * D,
+            "decode_bytes": lambda b: (params + head) * w4 + b * ctx * cfg["num_hidden_layers"] * 2 * G * D * 2}
+
+
+def _time(fn, sync, repeats: int) -> float:
+    fn()
+    sync()
+    best = float("inf")
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        fn()
+        sync()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def measure(engine, prompt, decode_steps: int, batches=(1, 4), free_running=None) -> dict:
+    """prefill seconds of `prompt` in one chunk and seconds per decode step at the batches given; the engine has max(batches) slots."""
+    out = {}
+
+    def prefill_once():
+        engine.begin(0)
+        engine.prefill(0, prompt, chunk=len(prompt))
+        engine.synchronize()
+        engine.release(0)
+
+    out["prefill_s"] = _time(prefill_once, engine.synchronize, 3)
+    for b in batches:
+        for s in range(b):
+            engine.begin(s)
+            engine.prefill(s, prompt, chunk=len(prompt))
+        run = (lambda: free_running(decode_steps, list(range(b)))) if free_running else (lambda: engine.decode(decode_steps, batch=b))
+        run()  # captures the step
+        engine.synchronize()
+        t0 = time.perf_counter()
+        run()
+        engine.synchronize()
+        out[f"decode_step_s_b{b}"] = (time.perf_counter() - t0) / decode_steps
+        for s in range(b):
+            engine.release(s)
+    return out
+
+
+def run(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, device: str = "cuda") -> dict:
+    import torch
+
+    from tiny_llm_hip.engine import DecodeEngine
+    from tiny_llm_hip.models import engine_for
+    from tiny_llm_hip.synthetic import synthetic_layer_list, synthetic_qwen3
+
+    rng = random.Random(seed)
+    results = []
+    for W in widths:
+        prompt = [rng.randrange(1, 32768) for _ in range(prompt_len)]
+        ctx = prompt_len + decode_steps
+        page = 128
+        pages = 4 * ((prompt_len + 3 * decode_steps) // page + 2)
+        row = {"width": W, "prompt_len": prompt_len, "decode_steps": decode_steps}
+        # the layer-list model
+        fcfg = fonapel_config(W)
+        model = synthetic_layer_list(fcfg, seed=seed, device=device)
+        eng = engine_for(model, dtype=torch.bfloat16, page_size=page, num_pages=pages, max_batch=4, max_pages_per_seq=pages // 4, max_prefill_rows=prompt_len)
+        try:
+            got = measure(eng, prompt, decode_steps, free_running=eng.decode_free_running)
+        finally:
+            eng.close()
+        del model
+        fc = fonapel_costs(fcfg, ctx)
+        row["fonapel"] = summarize(got, fc, prompt_len)
+        # Qwen3 W4A16 at equal sizes
+        qcfg = qwen3_config(W)
+        qmodel = synthetic_qwen3(qcfg, seed=seed, sigma=0.02, device=device)
+        qeng = DecodeEngine(qmodel, page_size=page, num_pages=pages, max_batch=4, max_pages_per_seq=pages // 4, max_prefill_rows=prompt_len)
+        try:
+            got = measure(qeng, prompt, decode_steps)
+        finally:
+            qeng.close()
+        del qmodel
+        row["qwen3_w4"] = summarize(got, qwen3_costs(qcfg, ctx), prompt_len)
+        for leg in ("prefill", "decode_b1", "decode_b4"):
+            a, b = row["fonapel"][leg]["roofline_fraction"], row["qwen3_w4"][leg]["roofline_fraction"]
+            row.setdefault("times_as_far_from_roofline", {})[leg] = round(b / a, 2) if a > 0 else None
+        results.append(row)
+        torch.cuda.empty_cache()
+    return {"bench": "layer_list_compare", "dtype": "bf16", "data": "synthetic", "roofline": {"hbm_bytes_per_s": HBM_BYTES_PER_S, "bf16_flops": BF16_FLOPS},
+            "results": results}
+
+
+def summarize(got: dict, costs: dict, prompt_len: int) -> dict:
+    flops = 2.0 * (costs["matrix_elems"] * prompt_len + costs["head_elems"]) + 2.0 * costs["attn_macs_per_pair"] * prompt_len * (prompt_len + 1) / 2
+    out = {"prefill": {"tokens_per_s": round(prompt_len / got["prefill_s"], 1), "ms": round(got["prefill_s"] * 1e3, 3), "tflops": round(flops / got["prefill_s"] / 1e12, 1),
+                       "roofline_fraction": round(flops / got["prefill_s"] / BF16_FLOPS, 4)}}
+    for b in (1, 4):
+        t = got[f"decode_step_s_b{b}"]
+        bytes_ = costs["decode_bytes"](b)
+        out[f"decode_b{b}"] = {"tokens_per_s": round(b / t, 1), "us_per_step": round(t * 1e6, 1), "gbytes_per_s": round(bytes_ / t / 1e9, 1),
+                               "roofline_fraction": round(bytes_ / t / HBM_BYTES_PER_S, 4)}
+    return out
+
+
+def main(widths, prompt_len=2048, decode_steps=64) -> None:
+    print(json.dumps(run(widths, prompt_len, decode_steps)), flush=True)

@@ -46,7 +46,7 @@ struct Run {
     int pass = -1;            // loop pass this run belongs to, -1 outside the loop
     bool enters_pass = false; // the loop-entry projection + pass offset come right before this run
     void *kpool = nullptr, *vpool = nullptr;      // attention: [pages, G, page, dim] / [pages, G, page, vdim] of the engine dtype
-    float *state = nullptr, *conv_state = nullptr; // delta: [slots, H, dim, vdim] / [slots, taps-1, C]
+    float *state = nullptr, *conv_state = nullptr; // delta: [slots, H, vdim, dim] / [slots, taps-1, C]
 };
 
 struct Meta {  // device int32 arrays of one step
@@ -166,28 +166,27 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
 }
 
 static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
-    // lanes per state column R and rows per lane RPT: key_dim <= RPT * R; a workgroup takes VB columns with VB * R <= 256 threads
-    int rpt = 8;
-    while (rpt < 128 && (L.dim + rpt - 1) / rpt > 16) rpt *= 2;
-    int R = 1;
-    while (R * rpt < L.dim) R *= 2;
-    TL_REQUIRE(R <= 64, "hybrid delta: key width above 8192 is not supported");
-    int VB = std::max(1, std::min(L.vdim, 256 / R));
-    const int threads = ((VB * R + 63) / 64) * 64;
-    int TB = (int)std::max<size_t>(1, std::min<size_t>(32, (48 * 1024 / 4) / (size_t)(2 * L.dim + VB + 2)));
-    const size_t lds = ((size_t)TB * (2 * L.dim + VB) + 2 * TB) * 4;
-    dim3 grid(L.heads, n_seqs, (L.vdim + VB - 1) / VB), block(threads);
+    // 16 lanes per state column, RPT key rows per lane: key_dim <= 16 RPT; a workgroup takes 16 columns
+    int rpt = 1;
+    while (16 * rpt < L.dim) rpt *= 2;
+    TL_REQUIRE(rpt <= 64, "hybrid delta: key width above 1024 is not supported");
+    const int DP = 16 * rpt;
+    const int TB = (int)std::max<size_t>(1, std::min<size_t>(32, (48 * 1024 / 4) / (size_t)(2 * DP + 18)));
+    const size_t lds = ((size_t)TB * (2 * DP + 16) + 2 * TB) * 4;
+    dim3 grid(L.heads, n_seqs, (L.vdim + 15) / 16), block(256);
     const int C = conv_channels(L);
     const int a0 = 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim, b0 = a0 + L.heads;
 #define HY_DELTA(RPT)                                                                                                                          \
     hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, lds, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
-                       L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim, R, VB, TB)
+                       L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim, TB)
     switch (rpt) {
+        case 1: HY_DELTA(1); break;
+        case 2: HY_DELTA(2); break;
+        case 4: HY_DELTA(4); break;
         case 8: HY_DELTA(8); break;
         case 16: HY_DELTA(16); break;
         case 32: HY_DELTA(32); break;
-        case 64: HY_DELTA(64); break;
-        default: HY_DELTA(128); break;
+        default: HY_DELTA(64); break;
     }
 #undef HY_DELTA
     TL_CHECK_LAUNCH("hybrid delta");
@@ -221,14 +220,18 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &r
     int HGB = 1;
     while (HGB < HG && HGB < 16) HGB *= 2;
     const int n_hblk = (HG + HGB - 1) / HGB, TQ = 64 / HGB;
-    const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
-    const size_t lds = (size_t)64 * ((4 * dk4 + 4) + (16 * vt_n + 4)) * 4;
+    const int vt_n = (L.vdim + 15) / 16;
+    const size_t lds = (size_t)64 * ((8 * ((L.dim + 7) / 8) + 4) + (16 * vt_n + 4)) * 4;
+    int page_shift = -1;
+    for (int b = 0; b < 30; ++b)
+        if ((1 << b) == c.page_size) page_shift = b;
+    const int vec_ok = L.dim % 8 == 0 && L.vdim % 8 == 0;
     auto kern = attn_tile_kernel<D, DK4, VT>;
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     dim3 grid((sh.max_len + TQ - 1) / TQ, L.kv_heads * n_hblk, sh.n_seqs * sh.n_splits);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)run.kpool, (const S *)run.vpool, m.seq_row0, m.seq_slot, m.row_pos,
                        e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.sink, HGB, n_hblk, sh.keys_per_split,
-                       sh.n_splits, gate, ldg, (S *)e->cat, ldo, e->part_acc, e->part_ml);
+                       sh.n_splits, gate, ldg, (S *)e->cat, ldo, e->part_acc, e->part_ml, page_shift, vec_ok);
     TL_CHECK_LAUNCH("hybrid attention tile");
     if (sh.n_splits > 1) {
         hipLaunchKernelGGL((attn_merge_kernel<D>), dim3(sh.rows, L.heads), dim3(64), 0, e->stream, e->part_acc, e->part_ml, sh.n_splits, L.heads, L.vdim, gate,
@@ -322,7 +325,7 @@ static int head_t(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
                        (const int32_t *)m.want_rows);
     TL_CHECK_LAUNCH("hybrid final norm");
     HY_TRY(linear_t<D>(e->hsel, c.width, c.head_dev, e->logits, c.vocab, n_want, c.vocab, c.width, 0, 1.f, nullptr, 0, e->stream));
-    hipLaunchKernelGGL(argmax_kernel, dim3(n_want), dim3(256), 0, e->stream, e->logits, c.vocab, e->argmax_dev, set_pending ? m.want_slot : (const int32_t *)nullptr,
+    hipLaunchKernelGGL(argmax_kernel, dim3(n_want), dim3(1024), 0, e->stream, e->logits, c.vocab, e->argmax_dev, set_pending ? m.want_slot : (const int32_t *)nullptr,
                        e->pending_dev);
     TL_CHECK_LAUNCH("hybrid argmax");
     return TL_OK;

@@ -383,10 +383,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                                                         const int32_t *seq_row0, const int32_t *seq_slot, const int32_t *row_pos,
                                                         const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
                                                         float scale, int sink, int HGB, int n_hblk, int keys_per_split, int n_splits, const float *gate,
-                                                        int ldg, typename D::storage *out, int ldo, float *part_acc, float *part_ml) {
+                                                        int ldg, typename D::storage *out, int ldo, float *part_acc, float *part_ml, int page_shift,
+                                                        int vec_ok) {
     using S = typename D::storage;
     extern __shared__ float smem[];
-    const int dk4 = (dim + 3) / 4, DKP = 4 * dk4 + 4, vt_n = (vdim + 15) / 16, VP = 16 * vt_n + 4;
+    const int dk4 = (dim + 3) / 4, DKP = 8 * ((dim + 7) / 8) + 4, vt_n = (vdim + 15) / 16, VP = 16 * vt_n + 4;
     float *Ks = smem;             // [64][DKP]
     float *Vs = smem + 64 * DKP;  // [64][VP]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, col = lane & 15;
@@ -413,32 +414,67 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
             const int d = 4 * kk + g4;
             qf[kk] = (row_ok && d < dim) ? qbuf[((size_t)trow * H + head) * dim + d] * scale : 0.f;
         }
+        // Staging: a tile is 64 (ck + cv) chunks of 8 elements; thread t owns chunks t, t + 256, ... -- the same (key, column) places in every
+        // tile, worked out once.  The next tile's chunks are loaded into registers before the current tile's products start, and go to LDS
+        // (as float32) after them: the loads' latency hides behind the matrix pipe.
+        constexpr int NIT = (DK4 / 2 + 2 * VT) / 4;
+        const int ck = (dim + 7) / 8, cv = 2 * vt_n, n_chunks = 64 * (ck + cv);
+        int place[NIT];  // key in tile | first column / 8 << 8 | is V << 24; -1: no chunk
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int q = tid + 256 * it;
+            if (q >= n_chunks) place[it] = -1;
+            else if (q < 64 * ck) place[it] = (q / ck) | ((q % ck) << 8);
+            else place[it] = ((q - 64 * ck) / cv) | (((q - 64 * ck) % cv) << 8) | (1 << 24);
+        }
+        S raw[NIT][8];
+        auto load_tile = [&](int kb) __attribute__((always_inline)) {
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int pl = place[it], j = kb + (pl & 255), c8 = 8 * ((pl >> 8) & 0xffff);
+                const bool is_v = (pl >> 24) & 1;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) raw[it][e] = (S)0;
+                if (pl >= 0 && j < k_end) {
+                    const int pg = page_shift >= 0 ? (j >> page_shift) : (j / page_size), in_pg = j - pg * page_size;
+                    const int wd = is_v ? vdim : dim;
+                    const S *src = (is_v ? vpool : kpool) + (((size_t)bt[pg] * G + kvh) * page_size + in_pg) * wd + c8;
+                    if (vec_ok) {
+                        if constexpr (sizeof(S) == 2) *reinterpret_cast<u32x4 *>(raw[it]) = *reinterpret_cast<const u32x4 *>(src);
+                        else {
+                            *reinterpret_cast<u32x4 *>(raw[it]) = *reinterpret_cast<const u32x4 *>(src);
+                            *reinterpret_cast<u32x4 *>(raw[it] + 4) = *reinterpret_cast<const u32x4 *>(src + 4);
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (c8 + e < wd) raw[it][e] = src[e];
+                    }
+                }
+            }
+        };
+        auto store_tile = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int pl = place[it];
+                if (pl < 0) continue;
+                float *dst = ((pl >> 24) & 1) ? Vs + (pl & 255) * VP + 8 * ((pl >> 8) & 0xffff) : Ks + (pl & 255) * DKP + 8 * ((pl >> 8) & 0xffff);
+                f32x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    lo[e] = D::to_float(raw[it][e]);
+                    hi[e] = D::to_float(raw[it][4 + e]);
+                }
+                *reinterpret_cast<f32x4 *>(dst) = lo;
+                *reinterpret_cast<f32x4 *>(dst + 4) = hi;
+            }
+        };
+        load_tile(k_begin);
         for (int kb = k_begin; kb < k_end; kb += 64) {
+            __syncthreads();  // every wave is done with the previous tile
+            store_tile();
             __syncthreads();
-            for (int i = tid; i < 64 * dk4; i += 256) {  // K tile -> float32
-                const int key = i / dk4, c4 = i % dk4, j = kb + key;
-                f32x4 v{0.f, 0.f, 0.f, 0.f};
-                if (j < k_end) {
-                    const S *src = kpool + (((size_t)bt[j / page_size] * G + kvh) * page_size + j % page_size) * dim + 4 * c4;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (4 * c4 + e < dim) v[e] = D::to_float(src[e]);
-                }
-                *reinterpret_cast<f32x4 *>(Ks + key * DKP + 4 * c4) = v;
-            }
-            const int v4 = 4 * vt_n;
-            for (int i = tid; i < 64 * v4; i += 256) {  // V tile -> float32
-                const int key = i / v4, c4 = i % v4, j = kb + key;
-                f32x4 v{0.f, 0.f, 0.f, 0.f};
-                if (j < k_end) {
-                    const S *src = vpool + (((size_t)bt[j / page_size] * G + kvh) * page_size + j % page_size) * vdim + 4 * c4;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (4 * c4 + e < vdim) v[e] = D::to_float(src[e]);
-                }
-                *reinterpret_cast<f32x4 *>(Vs + key * VP + 4 * c4) = v;
-            }
-            __syncthreads();
+            if (kb + 64 < k_end) load_tile(kb + 64);
             f32x4 sc[4];
             float m_tile = -INFINITY;
 #pragma unroll
@@ -585,99 +621,105 @@ __global__ void conv_state_kernel(const float *proj, int ldp, int taps, int C, c
 }
 
 // ---- gated delta rule, token by token ------------------------------------------------------------------------------------
-// grid (heads, sequences, column blocks of VB).  A thread holds RPT rows of one state column in registers; R = lanes per column
-// (a power of two <= 64, adjacent lanes), so key_dim <= RPT * R.  Per token:  S *= g;  u = beta (v - S^T k);  S += k u^T;  o = S^T q.
+// grid (heads, sequences, blocks of 16 state columns), 256 threads: 16 lanes (one DPP row) share a column of the state, each holding RPT
+// of its key_dim rows in registers (key_dim <= 16 RPT), so the two dot products of a token are RPT multiply-adds and one 16-lane DPP sum each.
+// Per token:  S *= g;  u = beta (v - S^T k);  S += k u^T;  o = S^T q.   State in memory: [slot, head, value_dim, key_dim] (a column's rows
+// are contiguous: the 16 lanes of a column read and write one run).
 // qkv: [rows, C] float32 after convolution + SiLU, q | k | v at 0 | G*dim | 2*G*dim.  q and k become unit vectors here
-// (x / sqrt(sum x^2 + unit_eps); q also * dim^-1/2).  ab: proj columns a0 + h (decay input) and b0 + h (beta input).
+// (x / sqrt(sum x^2 + unit_eps); q also * dim^-1/2).  proj columns a0 + h (decay input) and b0 + h (beta input).
 template <int RPT>
-__global__ void delta_kernel(const float *qkv, int C, const float *proj, int ldp, int a0, int b0, const float *a_log, const float *dt_bias,
-                             float unit_eps, const int32_t *seq_row0, const int32_t *seq_slot, float *state, float *obuf, int H, int G, int dim,
-                             int vdim, int R, int VB, int TB) {
+__global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, const float *proj, int ldp, int a0, int b0, const float *a_log,
+                                                    const float *dt_bias, float unit_eps, const int32_t *seq_row0, const int32_t *seq_slot, float *state,
+                                                    float *obuf, int H, int G, int dim, int vdim, int TB) {
+    constexpr int DP = 16 * RPT;  // padded key width: zeros behind dim
     extern __shared__ float smem[];
-    float *qs = smem;                 // [TB, dim]
-    float *ks = qs + (size_t)TB * dim;  // [TB, dim]
-    float *vs = ks + (size_t)TB * dim;  // [TB, VB]
-    float *gs = vs + (size_t)TB * VB;   // [TB]
-    float *bs = gs + TB;              // [TB]
-    const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * VB;
+    float *qs = smem;                  // [TB, DP]
+    float *ks = qs + (size_t)TB * DP;  // [TB, DP]
+    float *vs = ks + (size_t)TB * DP;  // [TB, 16]
+    float *gs = vs + (size_t)TB * 16;  // [TB]
+    float *bs = gs + TB;               // [TB]
+    const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * 16;
     const int kh = h / (H / G);
     const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
-    const int jl = tid / R, r = tid % R, j = j0 + jl;
-    const bool active = jl < VB && j < vdim;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int jl = tid >> 4, r = tid & 15, j = j0 + jl;
+    const bool active = j < vdim;
     float S[RPT];
-    float *sp = state + (((size_t)slot * H + h) * dim) * vdim;  // [dim, vdim]
+    float *sp = state + (((size_t)slot * H + h) * vdim + (active ? j : 0)) * dim + r * RPT;
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-        const int d = r * RPT + i;
-        S[i] = (active && d < dim) ? sp[(size_t)d * vdim + j] : 0.f;
-    }
+    for (int i = 0; i < RPT; ++i) S[i] = (active && r * RPT + i < dim) ? sp[i] : 0.f;
     const float decay_rate = -expf(a_log[h]), bias = dt_bias[h], qscale = 1.f / sqrtf((float)dim);
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int nt = min(TB, n - t0);
         __syncthreads();
-        for (int i = tid; i < nt * dim; i += blockDim.x) {
-            const int tt = i / dim, d = i % dim;
+        for (int i = tid; i < nt * DP; i += 256) {
+            const int tt = i / DP, d = i % DP;
             const float *row = qkv + (size_t)(r0 + t0 + tt) * C;
-            qs[i] = row[(size_t)kh * dim + d];
-            ks[i] = row[(size_t)(G + kh) * dim + d];
+            qs[i] = d < dim ? row[(size_t)kh * dim + d] : 0.f;
+            ks[i] = d < dim ? row[(size_t)(G + kh) * dim + d] : 0.f;
         }
-        for (int i = tid; i < nt * VB; i += blockDim.x) {
-            const int tt = i / VB, c = i % VB;
+        for (int i = tid; i < nt * 16; i += 256) {
+            const int tt = i >> 4, c = i & 15;
             vs[i] = (j0 + c < vdim) ? qkv[(size_t)(r0 + t0 + tt) * C + (size_t)2 * G * dim + (size_t)h * vdim + j0 + c] : 0.f;
         }
-        for (int tt = tid; tt < nt; tt += blockDim.x) {
+        for (int tt = tid; tt < nt; tt += 256) {
             const float *prow = proj + (size_t)(r0 + t0 + tt) * ldp;
             gs[tt] = expf(decay_rate * softplus_f(prow[a0 + h] + bias));
             bs[tt] = sigmoid_f(prow[b0 + h]);
         }
         __syncthreads();
-        for (int tt = wave; tt < nt; tt += nwaves) {  // unit vectors: one wave per token
+        for (int tt = wave; tt < nt; tt += 4) {  // unit vectors: one wave per token
             float sq = 0.f, sk = 0.f;
-            for (int d = lane; d < dim; d += 64) {
-                sq += qs[tt * dim + d] * qs[tt * dim + d];
-                sk += ks[tt * dim + d] * ks[tt * dim + d];
+            for (int d = lane; d < DP; d += 64) {
+                sq += qs[tt * DP + d] * qs[tt * DP + d];
+                sk += ks[tt * DP + d] * ks[tt * DP + d];
             }
             sq = wave_sum(sq);
             sk = wave_sum(sk);
             const float iq = qscale / sqrtf(sq + unit_eps), ik = 1.f / sqrtf(sk + unit_eps);
-            for (int d = lane; d < dim; d += 64) {
-                qs[tt * dim + d] *= iq;
-                ks[tt * dim + d] *= ik;
+            for (int d = lane; d < DP; d += 64) {
+                qs[tt * DP + d] *= iq;
+                ks[tt * DP + d] *= ik;
             }
         }
         __syncthreads();
-        if (active) {
-            for (int tt = 0; tt < nt; ++tt) {
-                const float g = gs[tt], b = bs[tt];
-                const float *kt = ks + tt * dim + r * RPT, *qt = qs + tt * dim + r * RPT;
-                float kv[RPT];
-                float dot = 0.f;
+        for (int tt = 0; tt < nt; ++tt) {  // (every lane runs the recurrence: the DPP sums want whole rows; idle columns store nothing)
+            const float g = gs[tt], b = bs[tt];
+            const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT;
+            float kv[RPT], qv[RPT];
+            if constexpr (RPT % 4 == 0) {
 #pragma unroll
-                for (int i = 0; i < RPT; ++i) {
-                    kv[i] = (r * RPT + i < dim) ? kt[i] : 0.f;
-                    S[i] *= g;
-                    dot += S[i] * kv[i];
-                }
-                for (int o = 1; o < R; o <<= 1) dot += __shfl_xor(dot, o, 64);
-                const float u = b * (vs[tt * VB + jl] - dot);
-                float od = 0.f;
+                for (int i = 0; i < RPT; i += 4) {
+                    const f32x4 k4 = *reinterpret_cast<const f32x4 *>(kt + i), q4 = *reinterpret_cast<const f32x4 *>(qt + i);
 #pragma unroll
-                for (int i = 0; i < RPT; ++i) {
-                    S[i] += kv[i] * u;
-                    od += S[i] * ((r * RPT + i < dim) ? qt[i] : 0.f);
+                    for (int e = 0; e < 4; ++e) kv[i + e] = k4[e], qv[i + e] = q4[e];
                 }
-                for (int o = 1; o < R; o <<= 1) od += __shfl_xor(od, o, 64);
-                if (r == 0) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
+            } else {
+#pragma unroll
+                for (int i = 0; i < RPT; ++i) kv[i] = kt[i], qv[i] = qt[i];
             }
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                S[i] *= g;
+                dot += S[i] * kv[i];
+            }
+            dot = group16_sum(dot);
+            const float u = b * (vs[tt * 16 + jl] - dot);
+            float od = 0.f;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                S[i] += kv[i] * u;
+                od += S[i] * qv[i];
+            }
+            od = group16_sum(od);
+            if (r == 0 && active) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
         }
     }
     if (active) {
 #pragma unroll
-        for (int i = 0; i < RPT; ++i) {
-            const int d = r * RPT + i;
-            if (d < dim) sp[(size_t)d * vdim + j] = S[i];
-        }
+        for (int i = 0; i < RPT; ++i)
+            if (r * RPT + i < dim) sp[i] = S[i];
     }
 }
 
@@ -704,39 +746,33 @@ __global__ void fill_kernel(float *p, size_t n, float v) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
 }
 // argmax of each logits row (first index wins on ties); also the next input token of the row's slot when slot_of_row is given
-__global__ __launch_bounds__(256) void argmax_kernel(const float *logits, int vocab, int32_t *out, const int32_t *slot_of_row, int32_t *pending) {
-    __shared__ float bv[4];
-    __shared__ int bi[4];
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *logits, int vocab, int32_t *out, const int32_t *slot_of_row, int32_t *pending) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
     const int r = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
     const float *row = logits + (size_t)r * vocab;
     float best = -INFINITY;
     int idx = 0x7fffffff;
-    for (int c = tid; c < vocab; c += 256) {
-        const float v = row[c];
-        if (v > best || (v == best && c < idx)) {
-            best = v;
-            idx = c;
+    auto take = [&](float v, int c) {
+        if (v > best || (v == best && c < idx)) best = v, idx = c;
+    };
+    if (vocab % 4 == 0) {
+        for (int c = 4 * tid; c < vocab; c += 4096) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(row + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) take(v[e], c + e);
         }
+    } else {
+        for (int c = tid; c < vocab; c += 1024) take(row[c], c);
     }
-    for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(best, o, 64);
-        const int oi = __shfl_xor(idx, o, 64);
-        if (ov > best || (ov == best && oi < idx)) {
-            best = ov;
-            idx = oi;
-        }
-    }
+    for (int o = 32; o > 0; o >>= 1) take(__shfl_xor(best, o, 64), __shfl_xor(idx, o, 64));
     if (lane == 0) {
         bv[tid >> 6] = best;
         bi[tid >> 6] = idx;
     }
     __syncthreads();
     if (tid == 0) {
-        for (int w = 1; w < 4; ++w)
-            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
-                best = bv[w];
-                idx = bi[w];
-            }
+        for (int w = 1; w < 16; ++w) take(bv[w], bi[w]);
         if (idx == 0x7fffffff) idx = 0;
         out[r] = idx;
         if (slot_of_row) pending[slot_of_row[r]] = idx;

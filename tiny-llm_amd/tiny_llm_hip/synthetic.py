@@ -123,3 +123,29 @@ def synthetic_qwen3(config: dict | str, seed: int = 0, sigma: float = 0.02, devi
     elif not cfg.get("tie_word_embeddings", True):
         out.lm_head = linear(cfg["vocab_size"], hs)
     return out
+
+
+def synthetic_layer_list(config: dict, seed: int = 0, device: str = "cuda", dtype: torch.dtype = torch.bfloat16) -> SimpleNamespace:
+    """A random-weight checkpoint object of a layer-list family (layer_list.FAMILIES by ``config["architecture"]``), as
+    ``loader.load_weights`` would return it: every tensor of the family's table, fan-in scaled normal matrices, small norm
+    offsets, drawn on ``device``."""
+    from .layer_list import FAMILIES
+
+    read_config, tensor_shapes = FAMILIES[config["architecture"]]
+    cfg = read_config(config)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    tensors = {}
+    for name, shape in tensor_shapes(cfg).items():
+        if len(shape) == 2 and not name.endswith(".conv") and name != "loop.step":
+            scale = 1.0 if name == "embed" else shape[1] ** -0.5
+        elif name.endswith("mix.norm"):
+            scale = 0.0
+        else:
+            scale = 0.1 if len(shape) == 1 else 0.5
+        t = torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * scale
+        if name.endswith("mix.norm"):
+            t = t + 1.0
+        tensors[name] = t.to(torch.bfloat16)
+    args = SimpleNamespace(vocab_size=cfg.vocab, hidden_size=cfg.width, num_hidden_layers=len(cfg.layers), architecture=cfg.family)
+    return SimpleNamespace(family=cfg.family, config=cfg, tensors=tensors, dtype=dtype, args=args)
