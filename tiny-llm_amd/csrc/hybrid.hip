@@ -220,8 +220,7 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &r
     int HGB = 1;
     while (HGB < HG && HGB < 16) HGB *= 2;
     const int n_hblk = (HG + HGB - 1) / HGB, TQ = 64 / HGB;
-    const int vt_n = (L.vdim + 15) / 16;
-    const size_t lds = (size_t)64 * ((8 * ((L.dim + 7) / 8) + 4) + (16 * vt_n + 4)) * 4;
+    const size_t lds = (size_t)64 * ((4 * DK4 + 4) + (16 * VT + 4)) * 4;
     int page_shift = -1;
     for (int b = 0; b < 30; ++b)
         if ((1 << b) == c.page_size) page_shift = b;

@@ -387,7 +387,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                                                         int vec_ok) {
     using S = typename D::storage;
     extern __shared__ float smem[];
-    const int dk4 = (dim + 3) / 4, DKP = 8 * ((dim + 7) / 8) + 4, vt_n = (vdim + 15) / 16, VP = 16 * vt_n + 4;
+    constexpr int DKP = 4 * DK4 + 4, VP = 16 * VT + 4;  // LDS rows as wide as the template: zeros behind dim / vdim, no guards in the product loops
     float *Ks = smem;             // [64][DKP]
     float *Vs = smem + 64 * DKP;  // [64][VP]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, col = lane & 15;
@@ -418,7 +418,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
         // tile, worked out once.  The next tile's chunks are loaded into registers before the current tile's products start, and go to LDS
         // (as float32) after them: the loads' latency hides behind the matrix pipe.
         constexpr int NIT = (DK4 / 2 + 2 * VT) / 4;
-        const int ck = (dim + 7) / 8, cv = 2 * vt_n, n_chunks = 64 * (ck + cv);
+        constexpr int ck = DK4 / 2, cv = 2 * VT, n_chunks = 64 * (ck + cv);
         int place[NIT];  // key in tile | first column / 8 << 8 | is V << 24; -1: no chunk
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
@@ -435,11 +435,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                 const bool is_v = (pl >> 24) & 1;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) raw[it][e] = (S)0;
-                if (pl >= 0 && j < k_end) {
+                if (pl >= 0 && j < k_end && c8 < (is_v ? vdim : dim)) {
                     const int pg = page_shift >= 0 ? (j >> page_shift) : (j / page_size), in_pg = j - pg * page_size;
                     const int wd = is_v ? vdim : dim;
                     const S *src = (is_v ? vpool : kpool) + (((size_t)bt[pg] * G + kvh) * page_size + in_pg) * wd + c8;
-                    if (vec_ok) {
+                    if (vec_ok) {  // (widths are multiples of 8: a chunk is whole or absent)
                         if constexpr (sizeof(S) == 2) *reinterpret_cast<u32x4 *>(raw[it]) = *reinterpret_cast<const u32x4 *>(src);
                         else {
                             *reinterpret_cast<u32x4 *>(raw[it]) = *reinterpret_cast<const u32x4 *>(src);
@@ -483,7 +483,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                 const float *kr = Ks + (16 * n + col) * DKP + g4;
 #pragma unroll
                 for (int kk = 0; kk < DK4; ++kk)
-                    if (kk < dk4) a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk], qf[kk], a4, 0, 0, 0);
+                    a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk], qf[kk], a4, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = kb + 16 * n + 4 * g4 + r;
@@ -520,7 +520,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                     const float *vr = Vs + (16 * n + 4 * g4 + r) * VP + col;
 #pragma unroll
                     for (int v = 0; v < VT; ++v)
-                        if (v < vt_n) o[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[n][r], o[v], 0, 0, 0);
+                        o[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[n][r], o[v], 0, 0, 0);
                 }
         }
     }
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int c = 16 * v + 4 * g4 + r;
-                if (v < vt_n && c < vdim) {
+                if (c < vdim) {
                     float val = o[v][r] * invl;
                     if (gate) val *= sigmoid_f(gate[(size_t)trow * ldg + (size_t)head * vdim + c]);
                     out[(size_t)trow * ldo + (size_t)head * vdim + c] = D::from_float(val);
@@ -545,7 +545,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int c = 16 * v + 4 * g4 + r;
-                if (v < vt_n && c < vdim) part_acc[pi * vdim + c] = o[v][r];
+                if (c < vdim) part_acc[pi * vdim + c] = o[v][r];
             }
         if (g4 == 0) {
             part_ml[2 * pi] = m_run;
