@@ -170,15 +170,12 @@ static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run 
     int rpt = 1;
     while (16 * rpt < L.dim) rpt *= 2;
     TL_REQUIRE(rpt <= 64, "hybrid delta: key width above 1024 is not supported");
-    const int DP = 16 * rpt;
-    const int TB = (int)std::max<size_t>(1, std::min<size_t>(32, (48 * 1024 / 4) / (size_t)(2 * DP + 18)));
-    const size_t lds = ((size_t)TB * (2 * DP + 16) + 2 * TB) * 4;
     dim3 grid(L.heads, n_seqs, (L.vdim + 15) / 16), block(256);
     const int C = conv_channels(L);
     const int a0 = 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim, b0 = a0 + L.heads;
 #define HY_DELTA(RPT)                                                                                                                          \
-    hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, lds, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
-                       L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim, TB)
+    hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, 0, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
+                       L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim)
     switch (rpt) {
         case 1: HY_DELTA(1); break;
         case 2: HY_DELTA(2); break;

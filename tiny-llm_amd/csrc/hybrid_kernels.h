@@ -630,18 +630,15 @@ __global__ void conv_state_kernel(const float *proj, int ldp, int taps, int C, c
 template <int RPT>
 __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, const float *proj, int ldp, int a0, int b0, const float *a_log,
                                                     const float *dt_bias, float unit_eps, const int32_t *seq_row0, const int32_t *seq_slot, float *state,
-                                                    float *obuf, int H, int G, int dim, int vdim, int TB) {
-    constexpr int DP = 16 * RPT;  // padded key width: zeros behind dim
-    extern __shared__ float smem[];
-    float *qs = smem;                  // [TB, DP]
-    float *ks = qs + (size_t)TB * DP;  // [TB, DP]
-    float *vs = ks + (size_t)TB * DP;  // [TB, 16]
-    float *gs = vs + (size_t)TB * 16;  // [TB]
-    float *bs = gs + TB;               // [TB]
+                                                    float *obuf, int H, int G, int dim, int vdim) {
+    constexpr int DP = 16 * RPT;                     // padded key width: zeros behind dim
+    constexpr int TB = RPT <= 8 ? 32 : 256 / RPT;    // tokens per LDS tile
+    constexpr int NIT = TB * DP / 256;               // q / k elements a thread stages per tile
+    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * 16], gs[TB], bs[TB];
     const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * 16;
     const int kh = h / (H / G);
     const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x;
     const int jl = tid >> 4, r = tid & 15, j = j0 + jl;
     const bool active = j < vdim;
     float S[RPT];
@@ -649,42 +646,52 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
 #pragma unroll
     for (int i = 0; i < RPT; ++i) S[i] = (active && r * RPT + i < dim) ? sp[i] : 0.f;
     const float decay_rate = -expf(a_log[h]), bias = dt_bias[h], qscale = 1.f / sqrtf((float)dim);
+    // The next tile's inputs travel through registers: loaded before the current tile's recurrence starts, written to LDS after it, so the
+    // loads' latency hides behind the token loop.
+    float rq[NIT], rk[NIT], rv[(TB * 16 + 255) / 256], ra = 0.f, rb = 0.f;
+    auto fetch = [&](int t0) __attribute__((always_inline)) {
+        const int nt = min(TB, n - t0);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int i = tid + 256 * it, tt = i / DP, d = i % DP;
+            const bool ok = tt < nt && d < dim;
+            const float *row = qkv + (size_t)(r0 + t0 + (ok ? tt : 0)) * C;
+            rq[it] = ok ? row[(size_t)kh * dim + d] : 0.f;
+            rk[it] = ok ? row[(size_t)(G + kh) * dim + d] : 0.f;
+        }
+#pragma unroll
+        for (int it = 0; it < (TB * 16 + 255) / 256; ++it) {
+            const int i = tid + 256 * it, tt = i >> 4, c = i & 15;
+            rv[it] = (tt < nt && j0 + c < vdim) ? qkv[(size_t)(r0 + t0 + tt) * C + (size_t)2 * G * dim + (size_t)h * vdim + j0 + c] : 0.f;
+        }
+        if (tid < nt) {
+            const float *prow = proj + (size_t)(r0 + t0 + tid) * ldp;
+            ra = prow[a0 + h];
+            rb = prow[b0 + h];
+        }
+    };
+    if (n > 0) fetch(0);
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int nt = min(TB, n - t0);
-        __syncthreads();
-        for (int i = tid; i < nt * DP; i += 256) {
-            const int tt = i / DP, d = i % DP;
-            const float *row = qkv + (size_t)(r0 + t0 + tt) * C;
-            qs[i] = d < dim ? row[(size_t)kh * dim + d] : 0.f;
-            ks[i] = d < dim ? row[(size_t)(G + kh) * dim + d] : 0.f;
+        __syncthreads();  // the previous tile's recurrence is done with the LDS
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            qs[tid + 256 * it] = rq[it];
+            ks[tid + 256 * it] = rk[it];
         }
-        for (int i = tid; i < nt * 16; i += 256) {
-            const int tt = i >> 4, c = i & 15;
-            vs[i] = (j0 + c < vdim) ? qkv[(size_t)(r0 + t0 + tt) * C + (size_t)2 * G * dim + (size_t)h * vdim + j0 + c] : 0.f;
-        }
-        for (int tt = tid; tt < nt; tt += 256) {
-            const float *prow = proj + (size_t)(r0 + t0 + tt) * ldp;
-            gs[tt] = expf(decay_rate * softplus_f(prow[a0 + h] + bias));
-            bs[tt] = sigmoid_f(prow[b0 + h]);
+#pragma unroll
+        for (int it = 0; it < (TB * 16 + 255) / 256; ++it)
+            if (tid + 256 * it < TB * 16) vs[tid + 256 * it] = rv[it];
+        if (tid < nt) {
+            gs[tid] = expf(decay_rate * softplus_f(ra + bias));
+            bs[tid] = sigmoid_f(rb);
         }
         __syncthreads();
-        for (int tt = wave; tt < nt; tt += 4) {  // unit vectors: one wave per token
-            float sq = 0.f, sk = 0.f;
-            for (int d = lane; d < DP; d += 64) {
-                sq += qs[tt * DP + d] * qs[tt * DP + d];
-                sk += ks[tt * DP + d] * ks[tt * DP + d];
-            }
-            sq = wave_sum(sq);
-            sk = wave_sum(sk);
-            const float iq = qscale / sqrtf(sq + unit_eps), ik = 1.f / sqrtf(sk + unit_eps);
-            for (int d = lane; d < DP; d += 64) {
-                qs[tt * DP + d] *= iq;
-                ks[tt * DP + d] *= ik;
-            }
-        }
-        __syncthreads();
-        for (int tt = 0; tt < nt; ++tt) {  // (every lane runs the recurrence: the DPP sums want whole rows; idle columns store nothing)
-            const float g = gs[tt], b = bs[tt];
+        if (t0 + TB < n) fetch(t0 + TB);
+        // every lane runs the recurrence (the DPP sums want whole rows; idle columns store nothing).  The 16 lanes of a column hold the whole
+        // key and query of the token between them, so they also form the two unit vectors.
+        for (int tt = 0; tt < nt; ++tt) {
+            const float g = gs[tt], b = bs[tt], vj = vs[tt * 16 + jl];
             const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT;
             float kv[RPT], qv[RPT];
             if constexpr (RPT % 4 == 0) {
@@ -698,21 +705,27 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
 #pragma unroll
                 for (int i = 0; i < RPT; ++i) kv[i] = kt[i], qv[i] = qt[i];
             }
-            float dot = 0.f;
+            float sk = 0.f, sq = 0.f, dot = 0.f;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
+                sk += kv[i] * kv[i];
+                sq += qv[i] * qv[i];
                 S[i] *= g;
                 dot += S[i] * kv[i];
             }
+            sk = group16_sum(sk);
+            sq = group16_sum(sq);
             dot = group16_sum(dot);
-            const float u = b * (vs[tt * 16 + jl] - dot);
+            const float ik = 1.f / sqrtf(sk + unit_eps), iq = qscale / sqrtf(sq + unit_eps);
+            const float u = b * (vj - dot * ik);  // S^T (k / |k|)
             float od = 0.f;
+            const float uk = u * ik;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                S[i] += kv[i] * u;
+                S[i] += kv[i] * uk;
                 od += S[i] * qv[i];
             }
-            od = group16_sum(od);
+            od = group16_sum(od) * iq;
             if (r == 0 && active) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
         }
     }
