@@ -634,7 +634,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
     constexpr int DP = 16 * RPT;                     // padded key width: zeros behind dim
     constexpr int TB = RPT <= 8 ? 32 : 256 / RPT;    // tokens per LDS tile
     constexpr int NIT = TB * DP / 256;               // q / k elements a thread stages per tile
-    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * 16], gs[TB], bs[TB];
+    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * 16], gs[TB], bs[TB], iqs[TB], iks[TB];
     const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * 16;
     const int kh = h / (H / G);
     const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
@@ -687,46 +687,69 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
             bs[tid] = sigmoid_f(rb);
         }
         __syncthreads();
+        {   // unit vectors: 256 / TB lanes per token form |q|^2 and |k|^2; the scales wait in LDS, outside the token loop's dependency chain
+            constexpr int LPT = 256 / TB;
+            const int tt = tid / LPT, sub = tid % LPT;
+            float sq = 0.f, sk = 0.f;
+            for (int d = sub; d < DP; d += LPT) {
+                sq += qs[tt * DP + d] * qs[tt * DP + d];
+                sk += ks[tt * DP + d] * ks[tt * DP + d];
+            }
+#pragma unroll
+            for (int o = 1; o < LPT; o <<= 1) {
+                sq += __shfl_xor(sq, o, 64);
+                sk += __shfl_xor(sk, o, 64);
+            }
+            if (sub == 0) {
+                iqs[tt] = qscale / sqrtf(sq + unit_eps);
+                iks[tt] = 1.f / sqrtf(sk + unit_eps);
+            }
+        }
+        __syncthreads();
         if (t0 + TB < n) fetch(t0 + TB);
-        // every lane runs the recurrence (the DPP sums want whole rows; idle columns store nothing).  The 16 lanes of a column hold the whole
-        // key and query of the token between them, so they also form the two unit vectors.
-        for (int tt = 0; tt < nt; ++tt) {
-            const float g = gs[tt], b = bs[tt], vj = vs[tt * 16 + jl];
+        // every lane runs the recurrence (the DPP sums want whole rows; idle columns store nothing); the next token's operands are read from
+        // LDS while the current token's chain runs
+        float g, b, vj, ik, iq, kv[RPT], qv[RPT];
+        auto read_token = [&](int tt, float &g_, float &b_, float &v_, float &ik_, float &iq_, float (&k_)[RPT], float (&q_)[RPT]) __attribute__((always_inline)) {
+            g_ = gs[tt], b_ = bs[tt], v_ = vs[tt * 16 + jl], ik_ = iks[tt], iq_ = iqs[tt];
             const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT;
-            float kv[RPT], qv[RPT];
             if constexpr (RPT % 4 == 0) {
 #pragma unroll
                 for (int i = 0; i < RPT; i += 4) {
                     const f32x4 k4 = *reinterpret_cast<const f32x4 *>(kt + i), q4 = *reinterpret_cast<const f32x4 *>(qt + i);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) kv[i + e] = k4[e], qv[i + e] = q4[e];
+                    for (int e = 0; e < 4; ++e) k_[i + e] = k4[e], q_[i + e] = q4[e];
                 }
             } else {
 #pragma unroll
-                for (int i = 0; i < RPT; ++i) kv[i] = kt[i], qv[i] = qt[i];
+                for (int i = 0; i < RPT; ++i) k_[i] = kt[i], q_[i] = qt[i];
             }
-            float sk = 0.f, sq = 0.f, dot = 0.f;
+        };
+        read_token(0, g, b, vj, ik, iq, kv, qv);
+        for (int tt = 0; tt < nt; ++tt) {
+            float ng, nb, nv, nik, niq, nk[RPT], nq[RPT];
+            read_token(tt + 1 < nt ? tt + 1 : tt, ng, nb, nv, nik, niq, nk, nq);
+            float dot0 = 0.f, dot1 = 0.f;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                sk += kv[i] * kv[i];
-                sq += qv[i] * qv[i];
                 S[i] *= g;
-                dot += S[i] * kv[i];
+                if (i & 1) dot1 += S[i] * kv[i];
+                else dot0 += S[i] * kv[i];
             }
-            sk = group16_sum(sk);
-            sq = group16_sum(sq);
-            dot = group16_sum(dot);
-            const float ik = 1.f / sqrtf(sk + unit_eps), iq = qscale / sqrtf(sq + unit_eps);
-            const float u = b * (vj - dot * ik);  // S^T (k / |k|)
-            float od = 0.f;
-            const float uk = u * ik;
+            const float dot = group16_sum(dot0 + dot1);
+            const float uk = b * (vj - dot * ik) * ik;  // u = beta (v - S^T k^), k^ = k / |k|;  S += k^ u^T = k (u / |k|)
+            float od0 = 0.f, od1 = 0.f;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
                 S[i] += kv[i] * uk;
-                od += S[i] * qv[i];
+                if (i & 1) od1 += S[i] * qv[i];
+                else od0 += S[i] * qv[i];
             }
-            od = group16_sum(od) * iq;
+            const float od = group16_sum(od0 + od1) * iq;
             if (r == 0 && active) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
+            g = ng, b = nb, vj = nv, ik = nik, iq = niq;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) kv[i] = nk[i], qv[i] = nq[i];
         }
     }
     if (active) {
