@@ -217,7 +217,7 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &r
     int HGB = 1;
     while (HGB < HG && HGB < 16) HGB *= 2;
     const int n_hblk = (HG + HGB - 1) / HGB, TQ = 64 / HGB;
-    const size_t lds = (size_t)64 * ((4 * DK4 + 4) + (16 * VT + 4)) * 4;
+    const size_t lds = (size_t)64 * ((sizeof(S) == 2 ? (4 * DK4 + 8) / 2 : 4 * DK4 + 4) + (16 * VT + 4)) * 4;  // K tile (bf16 as stored, or float32) + V tile (float32)
     int page_shift = -1;
     for (int b = 0; b < 30; ++b)
         if ((1 << b) == c.page_size) page_shift = b;
@@ -407,7 +407,7 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         const tl_hybrid_layer &L = e->layers[i];
         TL_REQUIRE(L.kind == TL_MIX_ATTENTION || L.kind == TL_MIX_DELTA, "hybrid_create: unknown mixer kind");
         TL_REQUIRE(L.heads > 0 && L.kv_heads > 0 && L.heads % L.kv_heads == 0, "hybrid_create: heads must be a positive multiple of kv_heads");
-        TL_REQUIRE(L.dim > 0 && L.dim <= 1024 && L.vdim > 0 && L.vdim <= 256, "hybrid_create: head widths: dim 1..1024, vdim 1..256");
+        TL_REQUIRE(L.dim > 0 && L.dim <= 1024 && L.vdim > 0 && L.vdim <= 512, "hybrid_create: head widths: dim 1..1024, vdim 1..512");
         TL_REQUIRE(L.w_in_dev && L.w_out_dev && L.norm_dev && L.ff >= 0, "hybrid_create: layer matrices and norm are required");
         if (L.kind == TL_MIX_ATTENTION) {
             TL_REQUIRE(L.rot_dims >= 0 && L.rot_dims % 2 == 0 && L.rot_dims <= L.dim, "hybrid_create: rot_dims must be even and at most dim");

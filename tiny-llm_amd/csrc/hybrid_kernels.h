@@ -324,7 +324,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
     for (int c = lane; c < dim; c += 64) qs[c] = qbuf[((size_t)t * H + h) * dim + c];
     __syncthreads();
     float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};  // vdim <= 256
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};  // vdim <= 512
     for (int kb = 0; kb <= pos; kb += 64) {
         const int j = kb + lane;
         float s = -INFINITY;
@@ -344,13 +344,13 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
         __syncthreads();
         const int cnt = min(64, pos - kb + 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] *= corr;
+        for (int i = 0; i < 8; ++i) acc[i] *= corr;
         for (int jj = 0; jj < cnt; ++jj) {
             const int jg = kb + jj;
             const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * G + g) * page_size + jg % page_size) * vdim;
             const float pj = ps[jj];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < 8; ++i) {
                 const int c = lane + i * 64;
                 if (c < vdim) acc[i] += pj * D::to_float(vr[c]);
             }
@@ -358,7 +358,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
     }
     const float invl = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 8; ++i) {
         const int c = lane + i * 64;
         if (c < vdim) {
             float o = acc[i] * invl;
@@ -387,7 +387,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                                                         int vec_ok) {
     using S = typename D::storage;
     extern __shared__ float smem[];
-    constexpr int DKP = 4 * DK4 + 4, VP = 16 * VT + 4;  // LDS rows as wide as the template: zeros behind dim / vdim, no guards in the product loops
+    // LDS rows as wide as the template: zeros behind dim / vdim, no guards in the product loops.  bfloat16 pages: the K tile stays bfloat16
+    // in LDS ([64][4 DK4 + 8] 16-bit elements) and S^T runs on v_mfma_f32_16x16x32_bf16 (q rounded to bfloat16 like every other input of a
+    // bfloat16 product, float32 sums, the scale applied to the float32 result); the weights and P V are float32 in either case.
+    constexpr bool KB16 = sizeof(S) == 2;
+    constexpr int DKP = KB16 ? (4 * DK4 + 8) / 2 : 4 * DK4 + 4, VP = 16 * VT + 4;  // (DKP in floats)
     float *Ks = smem;             // [64][DKP]
     float *Vs = smem + 64 * DKP;  // [64][VP]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g4 = lane >> 4, col = lane & 15;
@@ -408,11 +412,24 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 #pragma unroll
     for (int v = 0; v < VT; ++v) o[v] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (k_begin < k_end) {
-        float qf[DK4];
+        float qf[KB16 ? 1 : DK4];       // float32 pages: B operand of the 16x16x4 product, scale folded in
+        u32x4 qb[KB16 ? DK4 / 8 : 1];   // bfloat16 pages: B operand of the 16x16x32 product, 8 consecutive k per lane
+        if constexpr (KB16) {
 #pragma unroll
-        for (int kk = 0; kk < DK4; ++kk) {
-            const int d = 4 * kk + g4;
-            qf[kk] = (row_ok && d < dim) ? qbuf[((size_t)trow * H + head) * dim + d] * scale : 0.f;
+            for (int ks8 = 0; ks8 < DK4 / 8; ++ks8) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int d = 32 * ks8 + 8 * g4 + 2 * e;
+                    const float *qrow = qbuf + ((size_t)trow * H + head) * dim;
+                    qb[ks8][e] = BF16::pack2((row_ok && d < dim) ? qrow[d] : 0.f, (row_ok && d + 1 < dim) ? qrow[d + 1] : 0.f);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < DK4; ++kk) {
+                const int d = 4 * kk + g4;
+                qf[kk] = (row_ok && d < dim) ? qbuf[((size_t)trow * H + head) * dim + d] * scale : 0.f;
+            }
         }
         // Staging: a tile is 64 (ck + cv) chunks of 8 elements; thread t owns chunks t, t + 256, ... -- the same (key, column) places in every
         // tile, worked out once.  The next tile's chunks are loaded into registers before the current tile's products start, and go to LDS
@@ -458,6 +475,13 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
             for (int it = 0; it < NIT; ++it) {
                 const int pl = place[it];
                 if (pl < 0) continue;
+                if constexpr (KB16) {
+                    if (!((pl >> 24) & 1)) {  // a K chunk: 8 bfloat16 as they are
+                        *reinterpret_cast<u32x4 *>(reinterpret_cast<uint16_t *>(Ks) + (pl & 255) * (2 * DKP) + 8 * ((pl >> 8) & 0xffff)) =
+                            *reinterpret_cast<const u32x4 *>(raw[it]);
+                        continue;
+                    }
+                }
                 float *dst = ((pl >> 24) & 1) ? Vs + (pl & 255) * VP + 8 * ((pl >> 8) & 0xffff) : Ks + (pl & 255) * DKP + 8 * ((pl >> 8) & 0xffff);
                 f32x4 lo, hi;
 #pragma unroll
@@ -480,10 +504,20 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 #pragma unroll
             for (int n = 0; n < 4; ++n) {
                 f32x4 a4{0.f, 0.f, 0.f, 0.f};
-                const float *kr = Ks + (16 * n + col) * DKP + g4;
+                if constexpr (KB16) {
+                    const uint16_t *kr = reinterpret_cast<const uint16_t *>(Ks) + (16 * n + col) * (2 * DKP) + 8 * g4;
 #pragma unroll
-                for (int kk = 0; kk < DK4; ++kk)
-                    a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk], qf[kk], a4, 0, 0, 0);
+                    for (int ks8 = 0; ks8 < DK4 / 8; ++ks8) {
+                        const u32x4 ka = *reinterpret_cast<const u32x4 *>(kr + 32 * ks8);
+                        a4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ka), __builtin_bit_cast(bf16x8_t, qb[ks8]), a4, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) a4[r] *= scale;
+                } else {
+                    const float *kr = Ks + (16 * n + col) * DKP + g4;
+#pragma unroll
+                    for (int kk = 0; kk < DK4; ++kk) a4 = __builtin_amdgcn_mfma_f32_16x16x4f32(kr[4 * kk], qf[kk], a4, 0, 0, 0);
+                }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int j = kb + 16 * n + 4 * g4 + r;
