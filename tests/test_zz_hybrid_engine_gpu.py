@@ -75,11 +75,14 @@ MIXED = O.fonapel_config([O.delta_layer(), O.attention_layer(), O.attention_laye
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("layer", ["attention", "attention_ff", "delta", "delta_ff", "attention_full_rot", "attention_no_rot"])
+@pytest.mark.parametrize("layer", ["attention", "attention_ff", "delta", "delta_ff", "attention_full_rot", "attention_no_rot", "delta_wide_key",
+                                   "delta_many_columns"])
 def test_each_mixer_alone(layer, dtype):
     spec = {"attention": O.attention_layer(ff=0), "attention_ff": O.attention_layer(ff=48), "delta": O.delta_layer(ff=0),
             "delta_ff": O.delta_layer(ff=40), "attention_full_rot": O.attention_layer(dim=16, rot_dims=16, ff=0),
-            "attention_no_rot": O.attention_layer(rot_dims=0, ff=0)}[layer]
+            "attention_no_rot": O.attention_layer(rot_dims=0, ff=0),
+            "delta_wide_key": O.delta_layer(heads=2, kv_heads=1, dim=136, vdim=20, ff=0),         # a wave per state column
+            "delta_many_columns": O.delta_layer(heads=20, kv_heads=10, dim=72, vdim=128, ff=0)}[layer]  # 16 lanes per column, 8 rows each
     config = O.fonapel_config([spec])
     W = O.make_fonapel_weights(config, seed=1)
     toks = tokens_for(config, 37, seed=2)
@@ -123,7 +126,7 @@ def test_prefill_against_token_by_token(dtype):
         engine.close()
 
 
-@pytest.mark.parametrize("sizes", [[2], [3, 2, 7], [16], [15, 17, 1], [33, 2, 2, 40]])
+@pytest.mark.parametrize("sizes", [[2], [3, 2, 7], [16], [15, 17, 1], [33, 2, 2, 40], [70, 13]])
 def test_portions_of_several_sizes(sizes):
     W = O.make_fonapel_weights(MIXED, seed=7)
     toks = tokens_for(MIXED, 83, seed=8)

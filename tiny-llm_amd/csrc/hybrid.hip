@@ -166,24 +166,36 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
 }
 
 static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
-    // 16 lanes per state column, RPT key rows per lane: key_dim <= 16 RPT; a workgroup takes 16 columns
+    // LPC lanes per state column with RPT key rows each: key_dim <= LPC * RPT.  The token loop is a dependency chain, so a wave per column
+    // (the least work per wave) wins while the columns of the step put at most two waves on a SIMD; beyond that, and for narrow keys, a DPP
+    // row of 16 lanes per column
+    const int lpc = (L.dim > 64 && (long)L.heads * L.vdim * n_seqs <= 2 * 4 * (long)qmm3_num_cus()) ? 64 : 16;
     int rpt = 1;
-    while (16 * rpt < L.dim) rpt *= 2;
-    TL_REQUIRE(rpt <= 64, "hybrid delta: key width above 1024 is not supported");
-    dim3 grid(L.heads, n_seqs, (L.vdim + 15) / 16), block(256);
+    while (lpc * rpt < L.dim) rpt *= 2;
+    TL_REQUIRE(lpc * rpt <= 1024, "hybrid delta: key width above 1024 is not supported");
+    dim3 grid(L.heads, n_seqs, (L.vdim + 256 / lpc - 1) / (256 / lpc)), block(256);
     const int C = conv_channels(L);
     const int a0 = 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim, b0 = a0 + L.heads;
-#define HY_DELTA(RPT)                                                                                                                          \
-    hipLaunchKernelGGL((delta_kernel<RPT>), grid, block, 0, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
+#define HY_DELTA(RPT, LPC)                                                                                                                  \
+    hipLaunchKernelGGL((delta_kernel<RPT, LPC>), grid, block, 0, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
                        L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim)
-    switch (rpt) {
-        case 1: HY_DELTA(1); break;
-        case 2: HY_DELTA(2); break;
-        case 4: HY_DELTA(4); break;
-        case 8: HY_DELTA(8); break;
-        case 16: HY_DELTA(16); break;
-        case 32: HY_DELTA(32); break;
-        default: HY_DELTA(64); break;
+    if (lpc == 16) {
+        switch (rpt) {
+            case 1: HY_DELTA(1, 16); break;
+            case 2: HY_DELTA(2, 16); break;
+            case 4: HY_DELTA(4, 16); break;
+            case 8: HY_DELTA(8, 16); break;
+            case 16: HY_DELTA(16, 16); break;
+            case 32: HY_DELTA(32, 16); break;
+            default: HY_DELTA(64, 16); break;
+        }
+    } else {
+        switch (rpt) {
+            case 2: HY_DELTA(2, 64); break;
+            case 4: HY_DELTA(4, 64); break;
+            case 8: HY_DELTA(8, 64); break;
+            default: HY_DELTA(16, 64); break;
+        }
     }
 #undef HY_DELTA
     TL_CHECK_LAUNCH("hybrid delta");

@@ -655,25 +655,28 @@ __global__ void conv_state_kernel(const float *proj, int ldp, int taps, int C, c
 }
 
 // ---- gated delta rule, token by token ------------------------------------------------------------------------------------
-// grid (heads, sequences, blocks of 16 state columns), 256 threads: 16 lanes (one DPP row) share a column of the state, each holding RPT
-// of its key_dim rows in registers (key_dim <= 16 RPT), so the two dot products of a token are RPT multiply-adds and one 16-lane DPP sum each.
+// grid (heads, sequences, blocks of 256 / LPC state columns), 256 threads: LPC lanes (16 = one DPP row, or 64 = a wave) share a column of the
+// state, each holding RPT of its key_dim rows in registers (key_dim <= LPC RPT), so the two dot products of a token are RPT multiply-adds and
+// one DPP / wave sum each.  The token loop is a dependency chain: a wave per column (LPC 64) keeps the per-wave work smallest and puts two waves
+// on a SIMD at common sizes; LPC 16 serves narrow keys.
 // Per token:  S *= g;  u = beta (v - S^T k);  S += k u^T;  o = S^T q.   State in memory: [slot, head, value_dim, key_dim] (a column's rows
 // are contiguous: the 16 lanes of a column read and write one run).
 // qkv: [rows, C] float32 after convolution + SiLU, q | k | v at 0 | G*dim | 2*G*dim.  q and k become unit vectors here
 // (x / sqrt(sum x^2 + unit_eps); q also * dim^-1/2).  proj columns a0 + h (decay input) and b0 + h (beta input).
-template <int RPT>
+template <int RPT, int LPC>
 __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, const float *proj, int ldp, int a0, int b0, const float *a_log,
                                                     const float *dt_bias, float unit_eps, const int32_t *seq_row0, const int32_t *seq_slot, float *state,
                                                     float *obuf, int H, int G, int dim, int vdim) {
-    constexpr int DP = 16 * RPT;                     // padded key width: zeros behind dim
-    constexpr int TB = RPT <= 8 ? 32 : 256 / RPT;    // tokens per LDS tile
+    constexpr int DP = LPC * RPT;                    // padded key width: zeros behind dim
+    constexpr int CPB = 256 / LPC;                   // state columns of a workgroup
+    constexpr int TB = 4096 / DP < 32 ? 4096 / DP : 32;  // tokens per LDS tile (q and k tiles of 16 KB each at most)
     constexpr int NIT = TB * DP / 256;               // q / k elements a thread stages per tile
-    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * 16], gs[TB], bs[TB], iqs[TB], iks[TB];
-    const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * 16;
+    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * CPB], gs[TB], bs[TB], iqs[TB], iks[TB];
+    const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * CPB;
     const int kh = h / (H / G);
     const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
     const int tid = threadIdx.x;
-    const int jl = tid >> 4, r = tid & 15, j = j0 + jl;
+    const int jl = tid / LPC, r = tid % LPC, j = j0 + jl;
     const bool active = j < vdim;
     float S[RPT];
     float *sp = state + (((size_t)slot * H + h) * vdim + (active ? j : 0)) * dim + r * RPT;
@@ -682,7 +685,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
     const float decay_rate = -expf(a_log[h]), bias = dt_bias[h], qscale = 1.f / sqrtf((float)dim);
     // The next tile's inputs travel through registers: loaded before the current tile's recurrence starts, written to LDS after it, so the
     // loads' latency hides behind the token loop.
-    float rq[NIT], rk[NIT], rv[(TB * 16 + 255) / 256], ra = 0.f, rb = 0.f;
+    float rq[NIT], rk[NIT], rv[(TB * CPB + 255) / 256], ra = 0.f, rb = 0.f;
     auto fetch = [&](int t0) __attribute__((always_inline)) {
         const int nt = min(TB, n - t0);
 #pragma unroll
@@ -694,8 +697,8 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
             rk[it] = ok ? row[(size_t)(G + kh) * dim + d] : 0.f;
         }
 #pragma unroll
-        for (int it = 0; it < (TB * 16 + 255) / 256; ++it) {
-            const int i = tid + 256 * it, tt = i >> 4, c = i & 15;
+        for (int it = 0; it < (TB * CPB + 255) / 256; ++it) {
+            const int i = tid + 256 * it, tt = i / CPB, c = i % CPB;
             rv[it] = (tt < nt && j0 + c < vdim) ? qkv[(size_t)(r0 + t0 + tt) * C + (size_t)2 * G * dim + (size_t)h * vdim + j0 + c] : 0.f;
         }
         if (tid < nt) {
@@ -714,8 +717,8 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
             ks[tid + 256 * it] = rk[it];
         }
 #pragma unroll
-        for (int it = 0; it < (TB * 16 + 255) / 256; ++it)
-            if (tid + 256 * it < TB * 16) vs[tid + 256 * it] = rv[it];
+        for (int it = 0; it < (TB * CPB + 255) / 256; ++it)
+            if (tid + 256 * it < TB * CPB) vs[tid + 256 * it] = rv[it];
         if (tid < nt) {
             gs[tid] = expf(decay_rate * softplus_f(ra + bias));
             bs[tid] = sigmoid_f(rb);
@@ -745,7 +748,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
         // LDS while the current token's chain runs
         float g, b, vj, ik, iq, kv[RPT], qv[RPT];
         auto read_token = [&](int tt, float &g_, float &b_, float &v_, float &ik_, float &iq_, float (&k_)[RPT], float (&q_)[RPT]) __attribute__((always_inline)) {
-            g_ = gs[tt], b_ = bs[tt], v_ = vs[tt * 16 + jl], ik_ = iks[tt], iq_ = iqs[tt];
+            g_ = gs[tt], b_ = bs[tt], v_ = vs[tt * CPB + jl], ik_ = iks[tt], iq_ = iqs[tt];
             const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT;
             if constexpr (RPT % 4 == 0) {
 #pragma unroll
@@ -754,6 +757,9 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
 #pragma unroll
                     for (int e = 0; e < 4; ++e) k_[i + e] = k4[e], q_[i + e] = q4[e];
                 }
+            } else if constexpr (RPT == 2) {
+                const f32x2 k2 = *reinterpret_cast<const f32x2 *>(kt), q2 = *reinterpret_cast<const f32x2 *>(qt);
+                k_[0] = k2[0], k_[1] = k2[1], q_[0] = q2[0], q_[1] = q2[1];
             } else {
 #pragma unroll
                 for (int i = 0; i < RPT; ++i) k_[i] = kt[i], q_[i] = qt[i];
@@ -770,7 +776,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
                 if (i & 1) dot1 += S[i] * kv[i];
                 else dot0 += S[i] * kv[i];
             }
-            const float dot = group16_sum(dot0 + dot1);
+            const float dot = LPC == 16 ? group16_sum(dot0 + dot1) : wave_sum(dot0 + dot1);
             const float uk = b * (vj - dot * ik) * ik;  // u = beta (v - S^T k^), k^ = k / |k|;  S += k^ u^T = k (u / |k|)
             float od0 = 0.f, od1 = 0.f;
 #pragma unroll
@@ -779,7 +785,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
                 if (i & 1) od1 += S[i] * qv[i];
                 else od0 += S[i] * qv[i];
             }
-            const float od = group16_sum(od0 + od1) * iq;
+            const float od = (LPC == 16 ? group16_sum(od0 + od1) : wave_sum(od0 + od1)) * iq;
             if (r == 0 && active) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
             g = ng, b = nb, vj = nv, ik = nik, iq = niq;
 #pragma unroll
