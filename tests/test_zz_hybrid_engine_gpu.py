@@ -255,10 +255,10 @@ def test_far_keys_and_page_borders(needle_at, query):
         engine.close()
 
 
-@pytest.mark.parametrize("needle_at", [5, 255, 256, 511, 512, 640, 767, 768])
+@pytest.mark.parametrize("needle_at", [5, 63, 64, 127, 128, 255, 256, 511, 512, 640, 767, 768])
 def test_decoding_over_a_split_key_range(needle_at):
-    """From 512 keys on a single-token step splits a row's keys over workgroups (256 keys each) and merges the partial sums: the needle
-    sits at the splits' borders; the query is decoded alone, then greedy decoding goes on through the captured step."""
+    """From 256 keys on a single-token step splits a row's keys over workgroups (64 keys each, doubled beyond 64 splits) and merges the
+    partial sums: the needle sits at the splits' borders; the query is decoded alone, then greedy decoding goes on through the captured step."""
     config, W, A, B = _needle_model()
     toks = tokens_for(config, 800, seed=23, avoid=(A, B))
     toks[needle_at] = A
@@ -277,6 +277,25 @@ def test_decoding_over_a_split_key_range(needle_at):
         engine.decode_free_running(9, [0])       # feeds 790, then its own greedy ids
         engine.synchronize()
         assert engine.context_len(0) == 799
+        engine.release(0)
+    finally:
+        engine.close()
+
+
+@pytest.mark.parametrize("needle_at", [100, 4095, 4096, 4223])
+def test_decoding_over_more_keys_than_64_tiles(needle_at):
+    """Beyond 4,096 keys the splits take 128 keys each (two tiles per workgroup)."""
+    config, W, A, B = _needle_model()
+    toks = tokens_for(config, 4300, seed=26, avoid=(A, B))
+    toks[needle_at] = A
+    toks[-1] = B
+    want = O.fonapel_forward(config, W, toks)[-1]
+    engine = make_engine(config, W, page_size=64, num_pages=70, max_batch=1, max_prefill_rows=2048)
+    try:
+        engine.begin(0)
+        engine.prefill(0, toks[:-1], want_logits=False)
+        n = engine.step([(0, toks[-1:], [0])])
+        assert rel_err(engine.logits_host(n), want[None]) < TOL[torch.float32]
         engine.release(0)
     finally:
         engine.close()

@@ -207,12 +207,13 @@ struct StepShape {
     int n_splits = 1, keys_per_split = 1 << 30;  // attention: the key range of a row split over workgroups (decode steps over long contexts)
 };
 
-// how a step's attention splits the keys: only steps of single tokens, from 512 keys on; 256 keys per split, doubled until at most 64 splits
+// how a step's attention splits the keys: only steps of single tokens, from 256 keys on; one 64-key tile per split, doubled until at most 64
+// splits (a decode step is a few rows: its time is the chain of tiles a workgroup walks, so the chain is kept short and the chip full)
 static void plan_splits(StepShape &sh, int ctx_bound) {
     sh.n_splits = 1;
     sh.keys_per_split = 1 << 30;
-    if (sh.max_len != 1 || ctx_bound <= 512) return;
-    int kps = 256;
+    if (sh.max_len != 1 || ctx_bound <= 256) return;
+    int kps = 64;
     while ((ctx_bound + kps - 1) / kps > 64) kps *= 2;
     int n = 1;
     while (n * kps < ctx_bound) n *= 2;

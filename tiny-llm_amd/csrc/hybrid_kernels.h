@@ -588,26 +588,26 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
     }
 }
 
-// the splits of a row's key range put together: one wave per (row, query head)
+// the splits of a row's key range put together: one wave per (row, query head), n_splits <= 64.  Lane s owns split s for the maximum, the
+// sum and the weights exp(m_s - M); then the lanes turn to the value columns and walk the splits with those weights.
 template <typename D>
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float *part_acc, const float *part_ml, int n_splits, int H, int vdim, const float *gate,
                                                         int ldg, typename D::storage *out, int ldo) {
+    __shared__ float ws[64];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const size_t p0 = ((size_t)t * H + h) * n_splits;
-    float M = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) M = fmaxf(M, part_ml[2 * (p0 + s)]);
-    float L = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float m = part_ml[2 * (p0 + s)];
-        if (m != -INFINITY) L += part_ml[2 * (p0 + s) + 1] * expf(m - M);
-    }
+    const float m = lane < n_splits ? part_ml[2 * (p0 + lane)] : -INFINITY;
+    const float l = lane < n_splits ? part_ml[2 * (p0 + lane) + 1] : 0.f;
+    const float M = wave_max(m);
+    const float w = (m == -INFINITY) ? 0.f : expf(m - M);
+    const float L = wave_sum(l * w);
+    ws[lane] = w;
+    __syncthreads();
     const float invl = L > 0.f ? 1.f / L : 0.f;
     for (int c = lane; c < vdim; c += 64) {
         float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float m = part_ml[2 * (p0 + s)];
-            if (m != -INFINITY) acc += part_acc[(p0 + s) * vdim + c] * expf(m - M);
-        }
+#pragma unroll 8
+        for (int s = 0; s < n_splits; ++s) acc += part_acc[(p0 + s) * vdim + c] * ws[s];
         float val = acc * invl;
         if (gate) val *= sigmoid_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]);
         out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(val);
