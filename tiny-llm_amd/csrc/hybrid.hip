@@ -230,12 +230,15 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &r
     int HGB = 1;
     while (HGB < HG && HGB < 16) HGB *= 2;
     const int n_hblk = (HG + HGB - 1) / HGB, TQ = 64 / HGB;
-    const size_t lds = (size_t)64 * ((sizeof(S) == 2 ? (4 * DK4 + 8) / 2 : 4 * DK4 + 4) + (16 * VT + 4)) * 4;  // K tile (bf16 as stored, or float32) + V tile (float32)
+    const size_t lds_tiles = (size_t)64 * ((sizeof(S) == 2 ? (4 * DK4 + 8) / 2 : 4 * DK4 + 4) + (16 * VT + 4)) * 4;  // K tile (bf16 as stored, or float32) + V tile (float32)
     int page_shift = -1;
     for (int b = 0; b < 30; ++b)
         if ((1 << b) == c.page_size) page_shift = b;
     const int vec_ok = L.dim % 8 == 0 && L.vdim % 8 == 0;
-    auto kern = attn_tile_kernel<D, DK4, VT>;
+    // chunks whose rows fit one 16-row MFMA tile (decode steps): the four waves share the keys of a tile instead of the rows
+    const bool wsplit = sh.max_len * HGB <= 16;
+    const size_t lds = std::max(lds_tiles, (size_t)(128 + 4 * 64 * 4 * VT) * 4);
+    auto kern = wsplit ? attn_tile_kernel<D, DK4, VT, true> : attn_tile_kernel<D, DK4, VT, false>;
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     dim3 grid((sh.max_len + TQ - 1) / TQ, L.kv_heads * n_hblk, sh.n_seqs * sh.n_splits);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)run.kpool, (const S *)run.vpool, m.seq_row0, m.seq_slot, m.row_pos,

@@ -378,7 +378,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
 //                                 step r is key 4 g + r of the 16-key sub-tile (a sum does not care in which order its terms are paired)
 // Per query row (= per lane column) a running maximum and sum; the sink is their start value (0, 1).  The key range may be split over
 // gridDim.z (decode steps over long contexts): then unnormalised partial sums + (max, sum) go to part_* and attn_merge_kernel finishes.
-template <typename D, int DK4, int VT>
+template <typename D, int DK4, int VT, bool WSPLIT>
 __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
                                                         const int32_t *seq_row0, const int32_t *seq_slot, const int32_t *row_pos,
                                                         const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
@@ -404,10 +404,15 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
     const int k_end_tile = pos0 + min(t0 + TQ, len);  // keys the tile's last query row sees
     const int k_begin = split * keys_per_split, k_end = min(k_end_tile, (split + 1) * keys_per_split);
     // this lane's query row (column of the transposed products)
-    const int rho = wave * 16 + col, tl = rho / HGB, hb = hblk * HGB + rho % HGB;
+    // WSPLIT (a tile with at most 16 query rows, i.e. decode steps): every wave holds the SAME 16 rows and takes the 16 keys `wave` of each
+    // 64-key tile -- a quarter of the products per wave -- and the four partial (max, sum, O) sets are merged through LDS at the end
+    const int rho = (WSPLIT ? 0 : wave * 16) + col, tl = rho / HGB, hb = hblk * HGB + rho % HGB;
+    constexpr int NN = WSPLIT ? 1 : 4;  // 16-key sub-tiles a wave takes per tile
+    const int nb = WSPLIT ? wave : 0;
     const bool row_ok = t0 + tl < len && hb < HG;
     const int trow = r0 + t0 + tl, head = kvh * HG + hb, qpos = pos0 + t0 + tl;
-    float m_run = (sink && split == 0) ? 0.f : -INFINITY, l_run = (sink && split == 0) ? 1.f : 0.f;
+    const bool owns_sink = sink && split == 0 && (!WSPLIT || wave == 0);
+    float m_run = owns_sink ? 0.f : -INFINITY, l_run = owns_sink ? 1.f : 0.f;
     f32x4 o[VT];
 #pragma unroll
     for (int v = 0; v < VT; ++v) o[v] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -499,10 +504,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
             store_tile();
             __syncthreads();
             if (kb + 64 < k_end) load_tile(kb + 64);
-            f32x4 sc[4];
+            f32x4 sc[NN];
             float m_tile = -INFINITY;
 #pragma unroll
-            for (int n = 0; n < 4; ++n) {
+            for (int nn = 0; nn < NN; ++nn) {
+                const int n = nb + nn;
                 f32x4 a4{0.f, 0.f, 0.f, 0.f};
                 if constexpr (KB16) {
                     const uint16_t *kr = reinterpret_cast<const uint16_t *>(Ks) + (16 * n + col) * (2 * DKP) + 8 * g4;
@@ -524,7 +530,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                     a4[r] = (row_ok && j <= qpos && j < k_end) ? a4[r] : -INFINITY;
                     m_tile = fmaxf(m_tile, a4[r]);
                 }
-                sc[n] = a4;
+                sc[nn] = a4;
             }
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16, 64));
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
@@ -532,11 +538,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
             const float corr = (m_run == -INFINITY) ? 0.f : expf(m_run - m_new);
             float psum = 0.f;
 #pragma unroll
-            for (int n = 0; n < 4; ++n)
+            for (int nn = 0; nn < NN; ++nn)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float p = (sc[n][r] == -INFINITY) ? 0.f : expf(sc[n][r] - m_new);
-                    sc[n][r] = p;
+                    const float p = (sc[nn][r] == -INFINITY) ? 0.f : expf(sc[nn][r] - m_new);
+                    sc[nn][r] = p;
                     psum += p;
                 }
             psum += __shfl_xor(psum, 16, 64);
@@ -548,15 +554,48 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[v][r] *= corr;
 #pragma unroll
-            for (int n = 0; n < 4; ++n)
+            for (int nn = 0; nn < NN; ++nn)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float *vr = Vs + (16 * n + 4 * g4 + r) * VP + col;
+                    const float *vr = Vs + (16 * (nb + nn) + 4 * g4 + r) * VP + col;
 #pragma unroll
                     for (int v = 0; v < VT; ++v)
-                        o[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[n][r], o[v], 0, 0, 0);
+                        o[v] = __builtin_amdgcn_mfma_f32_16x16x4f32(vr[16 * v], sc[nn][r], o[v], 0, 0, 0);
                 }
         }
+    }
+    if constexpr (WSPLIT) {
+        // four waves, four partial sets of the same 16 rows: through LDS (the tiles are no longer needed) to wave 0
+        float *xm = smem, *xl = smem + 64, *xo = smem + 128;  // [4][16], [4][16], [4][64][4 VT]
+        __syncthreads();
+        if (g4 == 0) {
+            xm[wave * 16 + col] = m_run;
+            xl[wave * 16 + col] = l_run;
+        }
+#pragma unroll
+        for (int v = 0; v < VT; ++v) *reinterpret_cast<f32x4 *>(xo + ((size_t)(wave * 64 + lane) * VT + v) * 4) = o[v];
+        __syncthreads();
+        if (wave != 0) return;
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) M = fmaxf(M, xm[w * 16 + col]);
+        float L = 0.f;
+#pragma unroll
+        for (int v = 0; v < VT; ++v) o[v] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float mw = xm[w * 16 + col];
+            const float f = (mw == -INFINITY) ? 0.f : expf(mw - M);
+            L += xl[w * 16 + col] * f;
+#pragma unroll
+            for (int v = 0; v < VT; ++v) {
+                const f32x4 ow = *reinterpret_cast<const f32x4 *>(xo + ((size_t)(w * 64 + lane) * VT + v) * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[v][r] += ow[r] * f;
+            }
+        }
+        m_run = M;
+        l_run = L;
     }
     if (!row_ok) return;
     if (n_splits == 1) {
