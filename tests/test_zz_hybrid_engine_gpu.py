@@ -76,11 +76,12 @@ MIXED = O.fonapel_config([O.delta_layer(), O.attention_layer(), O.attention_laye
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("layer", ["attention", "attention_ff", "delta", "delta_ff", "attention_full_rot", "attention_no_rot", "delta_wide_key",
-                                   "delta_many_columns"])
+                                   "delta_many_columns", "attention_very_wide_head"])
 def test_each_mixer_alone(layer, dtype):
     spec = {"attention": O.attention_layer(ff=0), "attention_ff": O.attention_layer(ff=48), "delta": O.delta_layer(ff=0),
             "delta_ff": O.delta_layer(ff=40), "attention_full_rot": O.attention_layer(dim=16, rot_dims=16, ff=0),
             "attention_no_rot": O.attention_layer(rot_dims=0, ff=0),
+            "attention_very_wide_head": O.attention_layer(heads=2, kv_heads=1, dim=264, vdim=260, rot_dims=64, ff=0),  # beyond the tile kernel: a wave per row
             "delta_wide_key": O.delta_layer(heads=2, kv_heads=1, dim=136, vdim=20, ff=0),         # a wave per state column
             "delta_many_columns": O.delta_layer(heads=20, kv_heads=10, dim=72, vdim=128, ff=0)}[layer]  # 16 lanes per column, 8 rows each
     config = O.fonapel_config([spec])
@@ -89,6 +90,20 @@ def test_each_mixer_alone(layer, dtype):
     engine = make_engine(config, W, dtype)
     try:
         assert rel_err(whole(engine, toks), O.fonapel_forward(config, W, toks)) < TOL[dtype]
+    finally:
+        engine.close()
+
+
+def test_row_attention_twin_of_the_tile_kernel(monkeypatch):
+    """TL_HYBRID_ATTN_ROWS=1 runs every attention on the one-wave-per-row kernel; both forms must give the restatement's logits."""
+    W = O.make_fonapel_weights(MIXED, seed=27)
+    toks = tokens_for(MIXED, 90, seed=28)
+    want = O.fonapel_forward(MIXED, W, toks)
+    monkeypatch.setenv("TL_HYBRID_ATTN_ROWS", "1")
+    engine = make_engine(MIXED, W)
+    try:
+        assert rel_err(whole(engine, toks), want) < TOL[torch.float32]
+        assert rel_err(in_portions(engine, toks, [50, 1, 7]), want) < TOL[torch.float32]
     finally:
         engine.close()
 
