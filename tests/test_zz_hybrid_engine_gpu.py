@@ -76,12 +76,13 @@ MIXED = O.fonapel_config([O.delta_layer(), O.attention_layer(), O.attention_laye
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("layer", ["attention", "attention_ff", "delta", "delta_ff", "attention_full_rot", "attention_no_rot", "delta_wide_key",
-                                   "delta_many_columns", "attention_very_wide_head"])
+                                   "delta_many_columns", "attention_very_wide_head", "attention_large_group"])
 def test_each_mixer_alone(layer, dtype):
     spec = {"attention": O.attention_layer(ff=0), "attention_ff": O.attention_layer(ff=48), "delta": O.delta_layer(ff=0),
             "delta_ff": O.delta_layer(ff=40), "attention_full_rot": O.attention_layer(dim=16, rot_dims=16, ff=0),
             "attention_no_rot": O.attention_layer(rot_dims=0, ff=0),
             "attention_very_wide_head": O.attention_layer(heads=2, kv_heads=1, dim=264, vdim=260, rot_dims=64, ff=0),  # beyond the tile kernel: a wave per row
+            "attention_large_group": O.attention_layer(heads=24, kv_heads=1, dim=16, vdim=8, rot_dims=4, ff=0),  # 24 query heads on one K/V head: two blocks of 16
             "delta_wide_key": O.delta_layer(heads=2, kv_heads=1, dim=136, vdim=20, ff=0),         # a wave per state column
             "delta_many_columns": O.delta_layer(heads=20, kv_heads=10, dim=72, vdim=128, ff=0)}[layer]  # 16 lanes per column, 8 rows each
     config = O.fonapel_config([spec])
@@ -445,6 +446,45 @@ def test_checkpoint_directory_through_loader_registry_and_command_line(tmp_path,
     out = cli.main(["--model", str(tmp_path), "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "6", "--dtype", "float32",
                     "--sampler-temp", "1e-4", "--sampler-top-k", "1"])
     assert [int(t) for t in out.split()] == want
+
+
+def test_trace_replay_command_line(tmp_path):
+    """bin/trace_run on a checkpoint directory: steps as JSON lines on stdin, one packed pass per step, logits files and "done" lines out.
+    The first step is larger than the engine's row workspace (it is fed in portions); then two requests share steps, one ends and its
+    slot and pages serve a third."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from safetensors.torch import save_file
+
+    config, W, A, B = _needle_model()
+    model_dir, out_dir = tmp_path / "model", tmp_path / "out"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text(json.dumps(config))
+    save_file({k: torch.from_numpy(v).to(torch.bfloat16) for k, v in W.items()}, str(model_dir / "model.safetensors"))
+    long = tokens_for(config, 4200, seed=29, avoid=(A, B))
+    long[7], long[-1] = A, B
+    short = tokens_for(config, 30, seed=30)
+    third = tokens_for(config, 50, seed=31)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": long[:4150], "want": [0, 4149]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": long[4150:4199], "want": []}, {"id": "y", "tokens": short[:29], "want": [28]}], "end": []},
+             {"step": 2, "entries": [{"id": "y", "tokens": short[29:], "want": [0]}, {"id": "x", "tokens": long[4199:], "want": [0]}], "end": ["x"]},
+             {"step": 3, "entries": [], "end": []},
+             {"step": 4, "entries": [{"id": "z", "tokens": third, "want": [49, 3]}, {"id": "y", "tokens": [5], "want": []}], "end": ["y", "z"]}]
+    root = Path(__file__).resolve().parent.parent
+    run = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", "float32", "--out", str(out_dir),
+                          "--max-tokens", str(4224 + 64 + 64), "--slots", "2"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                         capture_output=True, text=True, timeout=110)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [l for l in run.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    ref_long, ref_short, ref_third = (O.fonapel_forward(config, W, t) for t in (long, short, third))
+    got = {i: np.fromfile(out_dir / f"{i}.f32", dtype="<f4").reshape(-1, config["vocab"]) for i in (0, 1, 2, 4)}
+    assert not (out_dir / "3.f32").exists()
+    assert rel_err(got[0], ref_long[[0, 4149]]) < TOL[torch.float32]
+    assert rel_err(got[1], ref_short[[28]]) < TOL[torch.float32]
+    assert rel_err(got[2], np.stack([ref_short[29], ref_long[4199]])) < TOL[torch.float32]
+    assert rel_err(got[4], ref_third[[49, 3]]) < TOL[torch.float32]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
