@@ -39,10 +39,11 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(scope="session")
 def built_libs():
-    """libtinyllm_hip.so (hipcc cross-compiles without a GPU) and the C oracle; built on demand."""
+    """libtinyllm_hip.so + libtinyllm_hybrid.so (hipcc cross-compiles without a GPU) and the C oracle; built on demand."""
     lib = ROOT / "tiny-llm_amd" / "extensions_hip" / "tiny_llm_ext_hip" / "libtinyllm_hip.so"
     ora = ROOT / "oracle" / "libqwen3_oracle.so"
-    if not lib.exists() or not ora.exists():
+    hyb = ROOT / "tiny-llm_amd" / "extensions_hip" / "tiny_llm_ext_hybrid" / "libtinyllm_hybrid.so"
+    if not lib.exists() or not ora.exists() or not hyb.exists():
         import __graft_entry__
 
         __graft_entry__.build()

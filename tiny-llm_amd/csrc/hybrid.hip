@@ -63,7 +63,6 @@ struct tl_hybrid {
     std::vector<float *> inv_freq;  // per layer (attention with rotary positions), device
     hipStream_t stream = nullptr;
     bool owns_stream = false;
-    int device = 0;
     std::unique_ptr<tl::PagePool> pool;
     bool table_dirty = true;
     int32_t *table_dev = nullptr;
@@ -77,7 +76,6 @@ struct tl_hybrid {
     int32_t *dmeta_dev = nullptr;                        // decode-loop metadata (its own copy: captured graphs point into it)
     int32_t *ctx_dev = nullptr, *pending_dev = nullptr, *argmax_dev = nullptr;
     tl::hy::Meta meta{}, dmeta{};
-    std::vector<int32_t> pending_host_valid;
     int last_rows = 0;
     // trace of the residual stream
     bool trace = false;
@@ -411,7 +409,6 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     auto e = std::make_unique<tl_hybrid>();
     e->cfg = c;
     e->layers.assign(layers, layers + c.num_layers);
-    HY_HIP(hipGetDevice(&e->device));
     if (stream) e->stream = (hipStream_t)stream;
     else {
         HY_HIP(hipDeviceSynchronize());

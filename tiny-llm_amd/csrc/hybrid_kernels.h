@@ -710,7 +710,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
     constexpr int CPB = 256 / LPC;                   // state columns of a workgroup
     constexpr int TB = 4096 / DP < 32 ? 4096 / DP : 32;  // tokens per LDS tile (q and k tiles of 16 KB each at most)
     constexpr int NIT = TB * DP / 256;               // q / k elements a thread stages per tile
-    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * CPB], gs[TB], bs[TB], iqs[TB], iks[TB];
+    __shared__ float qs[TB * DP], ks[TB * DP], vs[TB * CPB], gs[TB], bs[TB], iqs[TB], iks[TB], os[TB * CPB];
     const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * CPB;
     const int kh = h / (H / G);
     const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
@@ -825,10 +825,15 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
                 else od0 += S[i] * qv[i];
             }
             const float od = (LPC == 16 ? group16_sum(od0 + od1) : wave_sum(od0 + od1)) * iq;
-            if (r == 0 && active) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j] = od;
+            if (r == 0) os[tt * CPB + jl] = od;  // (read-outs leave the token loop through LDS: no global store inside the chain)
             g = ng, b = nb, vj = nv, ik = nik, iq = niq;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) kv[i] = nk[i], qv[i] = nq[i];
+        }
+        __syncthreads();
+        for (int i = tid; i < nt * CPB; i += 256) {
+            const int tt = i / CPB, c = i % CPB;
+            if (j0 + c < vdim) obuf[(size_t)(r0 + t0 + tt) * ((size_t)H * vdim) + (size_t)h * vdim + j0 + c] = os[i];
         }
     }
     if (active) {

@@ -163,15 +163,10 @@ class HybridEngine:
         if not slots:
             return
         arr = (ctypes.c_int * len(slots))(*slots)
-        if steps == 1:
+        for _ in range(steps):  # one captured step per call: the ids of every step are kept for read_tokens
             self._ext.check(self._lib.tl_hybrid_decode(self._h, len(slots), arr, 1, int(use_graph)))
             for s, tok in zip(slots, self.read_pending_slots(slots)):
                 self._produced.setdefault(s, []).append(tok)
-        else:
-            for _ in range(steps):  # the ids of every step are kept for read_tokens
-                self._ext.check(self._lib.tl_hybrid_decode(self._h, len(slots), arr, 1, int(use_graph)))
-                for s, tok in zip(slots, self.read_pending_slots(slots)):
-                    self._produced.setdefault(s, []).append(tok)
         self._rows = len(slots)
 
     def decode_free_running(self, steps: int, slots: Sequence[int], use_graph: bool = True) -> None:
