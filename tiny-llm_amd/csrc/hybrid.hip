@@ -164,10 +164,12 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
 }
 
 static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
-    // LPC lanes per state column with RPT key rows each: key_dim <= LPC * RPT.  The token loop is a dependency chain, so a wave per column
-    // (the least work per wave) wins while the columns of the step put at most two waves on a SIMD; beyond that, and for narrow keys, a DPP
-    // row of 16 lanes per column
-    const int lpc = (L.dim > 64 && (long)L.heads * L.vdim * n_seqs <= 2 * 4 * (long)qmm3_num_cus()) ? 64 : 16;
+    // LPC lanes per state column with RPT key rows each: key_dim <= LPC * RPT.  The token loop is a dependency chain whose cost per wave hardly
+    // depends on RPT, so the fewest lanes per column that still give every SIMD a wave: 64 while the step's columns are at most the SIMDs, then 32, then
+    // a DPP row of 16 (also for narrow keys)
+    const long cols = (long)L.heads * L.vdim * n_seqs, simds = 4 * (long)qmm3_num_cus();
+    int lpc = cols <= simds ? 64 : (cols <= 2 * simds ? 32 : 16);
+    while (lpc > 16 && lpc >= 2 * L.dim) lpc /= 2;  // no more lanes than key rows
     int rpt = 1;
     while (lpc * rpt < L.dim) rpt *= 2;
     TL_REQUIRE(lpc * rpt <= 1024, "hybrid delta: key width above 1024 is not supported");
@@ -177,24 +179,29 @@ static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run 
 #define HY_DELTA(RPT, LPC)                                                                                                                  \
     hipLaunchKernelGGL((delta_kernel<RPT, LPC>), grid, block, 0, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
                        L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim)
-    if (lpc == 16) {
+#define HY_DELTA_R(LPC)                          \
+    switch (rpt) {                               \
+        case 1: HY_DELTA(1, LPC); break;         \
+        case 2: HY_DELTA(2, LPC); break;         \
+        case 4: HY_DELTA(4, LPC); break;         \
+        case 8: HY_DELTA(8, LPC); break;         \
+        default: HY_DELTA(16, LPC); break;       \
+    }
+    if (lpc == 64) {
+        HY_DELTA_R(64)
+    } else if (lpc == 32) {
         switch (rpt) {
-            case 1: HY_DELTA(1, 16); break;
-            case 2: HY_DELTA(2, 16); break;
-            case 4: HY_DELTA(4, 16); break;
-            case 8: HY_DELTA(8, 16); break;
-            case 16: HY_DELTA(16, 16); break;
-            case 32: HY_DELTA(32, 16); break;
-            default: HY_DELTA(64, 16); break;
+            case 32: HY_DELTA(32, 32); break;
+            default: HY_DELTA_R(32)
         }
     } else {
         switch (rpt) {
-            case 2: HY_DELTA(2, 64); break;
-            case 4: HY_DELTA(4, 64); break;
-            case 8: HY_DELTA(8, 64); break;
-            default: HY_DELTA(16, 64); break;
+            case 32: HY_DELTA(32, 16); break;
+            case 64: HY_DELTA(64, 16); break;
+            default: HY_DELTA_R(16)
         }
     }
+#undef HY_DELTA_R
 #undef HY_DELTA
     TL_CHECK_LAUNCH("hybrid delta");
     return TL_OK;

@@ -694,7 +694,7 @@ __global__ void conv_state_kernel(const float *proj, int ldp, int taps, int C, c
 }
 
 // ---- gated delta rule, token by token ------------------------------------------------------------------------------------
-// grid (heads, sequences, blocks of 256 / LPC state columns), 256 threads: LPC lanes (16 = one DPP row, or 64 = a wave) share a column of the
+// grid (heads, sequences, blocks of 256 / LPC state columns), 256 threads: LPC lanes (16 = one DPP row, 32, or 64 = a wave) share a column of the
 // state, each holding RPT of its key_dim rows in registers (key_dim <= LPC RPT), so the two dot products of a token are RPT multiply-adds and
 // one DPP / wave sum each.  The token loop is a dependency chain: a wave per column (LPC 64) keeps the per-wave work smallest and puts two waves
 // on a SIMD at common sizes; LPC 16 serves narrow keys.
@@ -702,6 +702,14 @@ __global__ void conv_state_kernel(const float *proj, int ldp, int taps, int C, c
 // are contiguous: the 16 lanes of a column read and write one run).
 // qkv: [rows, C] float32 after convolution + SiLU, q | k | v at 0 | G*dim | 2*G*dim.  q and k become unit vectors here
 // (x / sqrt(sum x^2 + unit_eps); q also * dim^-1/2).  proj columns a0 + h (decay input) and b0 + h (beta input).
+// sum over the LPC adjacent lanes that share a state column (every lane of the wave takes part)
+template <int LPC>
+__device__ __forceinline__ float column_sum(float v, int lane) {
+    if constexpr (LPC == 64) return wave_sum(v);
+    v = group16_sum(v);
+    if constexpr (LPC == 32) v += lane_xor16(v, lane);
+    return v;
+}
 template <int RPT, int LPC>
 __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, const float *proj, int ldp, int a0, int b0, const float *a_log,
                                                     const float *dt_bias, float unit_eps, const int32_t *seq_row0, const int32_t *seq_slot, float *state,
@@ -815,7 +823,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
                 if (i & 1) dot1 += S[i] * kv[i];
                 else dot0 += S[i] * kv[i];
             }
-            const float dot = LPC == 16 ? group16_sum(dot0 + dot1) : wave_sum(dot0 + dot1);
+            const float dot = column_sum<LPC>(dot0 + dot1, tid);
             const float uk = b * (vj - dot * ik) * ik;  // u = beta (v - S^T k^), k^ = k / |k|;  S += k^ u^T = k (u / |k|)
             float od0 = 0.f, od1 = 0.f;
 #pragma unroll
@@ -824,7 +832,7 @@ __global__ __launch_bounds__(256) void delta_kernel(const float *qkv, int C, con
                 if (i & 1) od1 += S[i] * qv[i];
                 else od0 += S[i] * qv[i];
             }
-            const float od = (LPC == 16 ? group16_sum(od0 + od1) : wave_sum(od0 + od1)) * iq;
+            const float od = column_sum<LPC>(od0 + od1, tid) * iq;
             if (r == 0) os[tt * CPB + jl] = od;  // (read-outs leave the token loop through LDS: no global store inside the chain)
             g = ng, b = nb, vj = nv, ik = nik, iq = niq;
 #pragma unroll
