@@ -15,6 +15,28 @@
  *                      towards the new value along the new key and is read with the query; q/k/v pass a short
  *                      causal depthwise convolution + SiLU first.  The state and the convolution's last inputs
  *                      live in one state slot per sequence.
+ *   TL_MIX_LINREC      linear recurrence with a decaying matrix state per head, S <- diag(a_t) S + b_t k_t v_t^T,
+ *                      o_t = S^T q_t (q scaled by dim^-1/2).  rec_kind TL_REC_CHANNEL: a decay per key channel,
+ *                      sigmoid(z)^(1/tau) with z from a low-rank pair of projections plus a bias, b = 1 (gated linear
+ *                      attention); the read-out is RMS-normed per head with a [vdim] weight and gated by SiLU.
+ *                      rec_kind TL_REC_EXPGATE: exponential input and forget gates per head, capped by
+ *                      cap tanh(x / cap), with a running maximum m (starting at 0) that keeps them in range, and a
+ *                      normaliser n_t = a n + b k: o / (max(|n.q|, e^-m) + 1e-6) (the matrix memory of xLSTM); the
+ *                      read-out is unit-RMS per head, times a [heads*vdim] weight, gated by a sigmoid.
+ *                      State (and m) live in the state slot of the sequence.
+ *   TL_MIX_LATENT      latent attention: queries through a normed low-rank latent; keys and values are per-head
+ *                      projections (W_uk, W_uv) of ONE normed latent c [kv_rank] per token, plus one rotated key part
+ *                      [rot_dim] shared by all heads; only (c | rotated part) is cached, one row per token.  The engine
+ *                      runs it in absorbed form: q_h' = W_uk,h^T q_h, scores (q_h' . c + q_rot . k_rot) * scale, output
+ *                      W_uv,h (sum_j p_j c_j) -- one K/V head of width kv_rank + rot_dim whose values are its leading
+ *                      kv_rank columns.  Rotation frequencies may be rescaled (YaRN: rot_factor > 0).  kv_from >= 0: the
+ *                      layer has no latent projection of its own and reads the pages of that earlier layer.
+ *
+ * Block forms: parallel_block 1 is x += m (mixer(h) + ff(h)) with one norm; 0 is the sequential pre-norm block
+ * x += ls1 * mixer(norm1 x); x += ls2 * ff(norm2 x) with optional per-channel scales ls1 / ls2.  Norms: RMS or
+ * Dynamic Tanh (tanh(alpha x) w + b).  Feed-forward kinds: W_down act(W_up h), W_down (act(W_gate h) * W_up h), or a
+ * mixture of experts (softmax router with a selection-only correction, groups of neighbouring experts, identity
+ * experts, a gated shared expert).
  *
  * A contiguous range of layers may be repeated ("loop"): each pass has its own K/V pages / state slots, and is
  * entered through a [width, 2 width] projection of the running stream beside the embedding output plus a per-pass
@@ -43,15 +65,28 @@ extern "C" {
 
 typedef struct tl_hybrid tl_hybrid;
 
-enum { TL_MIX_ATTENTION = 0, TL_MIX_DELTA = 1 };
+enum { TL_MIX_ATTENTION = 0, TL_MIX_DELTA = 1, TL_MIX_LINREC = 2, TL_MIX_LATENT = 3 };
+enum { TL_REC_CHANNEL = 0, TL_REC_EXPGATE = 1 };
+enum { TL_NORM_RMS = 0, TL_NORM_DYT = 1 };
+enum { TL_FF_PLAIN = 0, TL_FF_GATED = 1, TL_FF_MOE = 2 };
+enum { TL_ACT_GELU_ERF = 0, TL_ACT_GELU_TANH = 1, TL_ACT_SILU = 2, TL_ACT_RELU2 = 3 };
 enum { TL_HY_F32 = 0, TL_HY_BF16 = 2 }; /* the values of tl_dtype in tinyllm_hip.h */
 
 /* One layer.  Matrices are [out, in] row-major in the engine's dtype; vectors are float32.
  * w_in: every projection that reads the normed input, rows concatenated in this order:
  *   attention: q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim) | gate (heads*vdim, if gated) | up (ff, if ff > 0)
  *   delta:     q (kv_heads*dim) | k (kv_heads*dim) | v (heads*vdim) | gate (heads*vdim) | a (heads) | b (heads) | up (ff)
+ *   linrec:    q (heads*dim) | k (heads*dim) | v (heads*vdim) | gate (heads*vdim) | expgate: i (heads) | f (heads)
+ *                                                                                    | channel: a1 (a_rank)
+ *   latent:    dq (q_rank) | dkv (kv_rank + rot_dim, unless kv_from >= 0) | gate (heads*vdim)
  * w_out: [width, heads*vdim + ff]: the mixer's output projection beside the feed-forward's down projection, so
- *   one product yields mixer(h) + ff(h). */
+ *   one product yields mixer(h) + ff(h).
+ * Sequential block (parallel_block 0): w_in / w_out hold the mixer's rows / columns only; the feed-forward reads
+ *   norm2 through w_in2 and returns through w_out2:
+ *   plain: up (ff)                   -> w_out2 [width, ff]
+ *   gated: gate (ff) | up (ff)       -> w_out2 [width, ff]
+ *   moe:   router (experts + identity) | shared gate (1) | shared up (shared_ff) | expert 0 up (expert_ff) | expert 1 up ...
+ *                                    -> w_out2 [width, shared_ff + experts * expert_ff]: shared down | expert 0 down | ... */
 typedef struct tl_hybrid_layer {
     int kind;
     int heads, kv_heads, dim, vdim;
@@ -73,13 +108,38 @@ typedef struct tl_hybrid_layer {
     const float *a_log_dev, *dt_bias_dev; /* [heads] */
     const float *out_norm_dev;            /* [vdim] */
     float unit_eps;         /* q, k -> x / sqrt(sum x^2 + unit_eps) */
+    /* norms and the sequential block */
+    int norm_kind;          /* TL_NORM_RMS / TL_NORM_DYT, both norms of the layer */
+    float norm_alpha, norm2_alpha;                /* Dynamic Tanh: the scalar inside the tanh */
+    const float *norm_bias_dev, *norm2_bias_dev;  /* Dynamic Tanh: [width] */
+    const float *norm2_dev;                       /* [width] the feed-forward's pre-norm (sequential block) */
+    const void *w_in2_dev, *w_out2_dev;           /* the feed-forward's matrices (sequential block) */
+    const float *ls1_dev, *ls2_dev;               /* [width] per-channel scale of the mixer's / feed-forward's result; NULL: none */
+    int ff_kind;            /* TL_FF_* */
+    /* mixture of experts (ff_kind TL_FF_MOE; ff = shared_ff + experts * expert_ff) */
+    int experts, identity, top, groups, keep, expert_ff, shared_ff;
+    const float *correction_dev;                  /* [experts + identity] added to the scores for the selection only */
+    /* linear recurrence */
+    int rec_kind;           /* TL_REC_* */
+    float gate_cap, tau;
+    int a_rank;             /* channel decay: rank of the projection pair */
+    const void *a2_dev;     /* [heads*dim, a_rank] engine dtype */
+    const float *a2_bias_dev;                     /* [heads*dim] */
+    const float *i_bias_dev, *f_bias_dev;         /* [heads] */
+    /* latent attention (out_norm_dev is not used; heads share one K/V head) */
+    int q_rank, kv_rank, rot_dim, kv_from;        /* kv_from: layer index whose pages are read, -1: the layer's own */
+    const float *dq_norm_dev, *dkv_norm_dev;      /* [q_rank], [kv_rank] */
+    const void *uq_dev;     /* [heads*(dim + rot_dim), q_rank] */
+    const void *uk_t_dev;   /* [heads, kv_rank, dim]: W_uk of every head transposed */
+    const void *uv_dev;     /* [heads, vdim, kv_rank] */
+    float rot_factor, rot_original, rot_fast, rot_slow; /* rot_factor <= 0: plain frequencies */
 } tl_hybrid_layer;
 
 typedef struct tl_hybrid_config {
     int dtype;              /* TL_HY_BF16 or TL_HY_F32 */
     int width, vocab, num_layers;
     float norm_eps, residual_mult;
-    int parallel_block;     /* 1: x += m * (mixer(h) + ff(h)) with one norm (the only form so far) */
+    int parallel_block;     /* 1: x += m * (mixer(h) + ff(h)) with one norm; 0: x += m ls1 mixer(norm1 x), then x += m ls2 ff(norm2 x) */
     int loop_start, loop_stop, loop_times; /* loop_times <= 1 or start == stop: no loop */
     const void *loop_in_dev;    /* [width, 2*width], stream first */
     const float *loop_step_dev; /* [loop_times, width] */
@@ -87,6 +147,10 @@ typedef struct tl_hybrid_config {
     const float *final_norm_dev;
     float final_norm_offset;
     const void *head_dev;       /* [vocab, width] */
+    float embed_scale;          /* x = embed[token] * embed_scale (0 is read as 1) */
+    int final_norm_kind;        /* TL_NORM_* */
+    float final_norm_alpha;
+    const float *final_norm_bias_dev;
     int page_size, num_pages, max_slots, max_pages_per_seq, max_rows;
 } tl_hybrid_config;
 

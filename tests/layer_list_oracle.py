@@ -192,3 +192,191 @@ def fonapel_config(layers, width=64, vocab=101, loop=None, eps=1e-5, residual_mu
     if loop:
         cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
     return cfg
+
+
+# ---- Zefapel: sequential pre-norm layers (Dynamic Tanh norms, layer scale), mixers "mlstm" / "gla" / "latent_attention", dense or
+# ---- mixture-of-experts feed-forward.  Same conventions: float64, whole sequences, one function per mechanism. -------------------
+
+def dyt_norm(x, alpha, weight, bias):
+    """tanh(alpha x) * weight + bias (no statistics of x)."""
+    return np.tanh(alpha * x) * weight + bias
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + np.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+
+
+def log_sigmoid(z):
+    return -softplus(-z)
+
+
+def scaled_frequencies(dims, base, scaling=None):
+    """Rotation frequencies f_i = base^(-2i/dims), i < dims/2, and the factor on cos / sin.  With ``scaling`` (factor, original,
+    fast, slow): dimensions that turn fewer than `slow` times over `original` positions are slowed by `factor`, those that turn
+    more than `fast` times are kept, a linear ramp in between; cos and sin grow by 0.1 ln(factor) + 1."""
+    f = np.array([base ** (-2.0 * i / dims) for i in range(dims // 2)])
+    if not scaling:
+        return f, 1.0
+
+    def where(turns):
+        return dims * math.log(scaling["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+    lo = max(math.floor(where(scaling["fast"])), 0)
+    hi = min(math.ceil(where(scaling["slow"])), dims - 1)
+    ramp = np.clip((np.arange(dims // 2) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    return f / scaling["factor"] * ramp + f * (1.0 - ramp), 0.1 * math.log(scaling["factor"]) + 1.0
+
+
+def rotate_pairs_by(z, positions, freqs, mult=1.0):
+    """z [L, ..., >= 2 len(freqs)]: the pair (2i, 2i+1) at position p turns by p * freqs[i]; cos and sin times ``mult``."""
+    out = z.copy()
+    for i, f in enumerate(freqs):
+        shape = (-1,) + (1,) * (z.ndim - 2)
+        c, s = (np.cos(positions * f) * mult).reshape(shape), (np.sin(positions * f) * mult).reshape(shape)
+        u, v = z[..., 2 * i], z[..., 2 * i + 1]
+        out[..., 2 * i] = u * c - v * s
+        out[..., 2 * i + 1] = v * c + u * s
+    return out
+
+
+def matrix_memory(q, k, v, log_i, log_f):
+    """mLSTM cell.  q, k [L, H, D] (q already scaled), v [L, H, V], log_i / log_f [L, H] (log input and forget gates).  Per head,
+    with a running maximum m that starts at 0:  m' = max(f + m, i);  S <- e^(f + m - m') S + e^(i - m') k v^T;  n likewise with k;
+    o = S^T q / (max(|n.q|, e^(-m')) + 1e-6)."""
+    L, H, V = v.shape
+    D = q.shape[2]
+    out = np.zeros((L, H, V))
+    for h in range(H):
+        S, n, m = np.zeros((D, V)), np.zeros(D), 0.0
+        for t in range(L):
+            m_new = max(log_f[t, h] + m, log_i[t, h])
+            a, b = math.exp(log_f[t, h] + m - m_new), math.exp(log_i[t, h] - m_new)
+            S = a * S + b * np.outer(k[t, h], v[t, h])
+            n = a * n + b * k[t, h]
+            m = m_new
+            out[t, h] = S.T @ q[t, h] / (max(abs(n @ q[t, h]), math.exp(-m)) + 1e-6)
+    return out
+
+
+def gated_linear_attention(q, k, v, alpha):
+    """q, k, alpha [L, H, D], v [L, H, V].  Per head: S <- diag(alpha_t) S + k_t v_t^T;  o_t = S^T q_t."""
+    L, H, V = v.shape
+    D = q.shape[2]
+    out = np.zeros((L, H, V))
+    for h in range(H):
+        S = np.zeros((D, V))
+        for t in range(L):
+            S = alpha[t, h][:, None] * S + np.outer(k[t, h], v[t, h])
+            out[t, h] = S.T @ q[t, h]
+    return out
+
+
+def causal_softmax_attention(q, k, v, scale):
+    """q [L, H, D], k [L, H, D], v [L, H, V]: row i sees keys j <= i; ordinary softmax."""
+    L, H, _ = q.shape
+    out = np.zeros((L, H, v.shape[2]))
+    for h in range(H):
+        for i in range(L):
+            s = (k[: i + 1, h] @ q[i, h]) * scale
+            e = np.exp(s - s.max())
+            out[i, h] = (e / e.sum()) @ v[: i + 1, h]
+    return out
+
+
+def route(z, correction, top, groups, keep):
+    """z [E] router logits.  Scores s = softmax(z); choice = s + correction; only experts of the `keep` groups (of `groups`
+    equal runs of neighbours) with the largest group maximum of choice can be taken; the `top` largest choices win; weights are
+    their s.  Returns {expert: weight}."""
+    e = np.exp(z - z.max())
+    s = e / e.sum()
+    choice = s + correction
+    E = len(z)
+    per = E // groups
+    gmax = [choice[g * per:(g + 1) * per].max() for g in range(groups)]
+    kept = sorted(range(groups), key=lambda g: (-gmax[g], g))[:keep]
+    allowed = [j for j in range(E) if j // per in kept]
+    chosen = sorted(allowed, key=lambda j: (-choice[j], j))[:top]
+    return {j: s[j] for j in chosen}
+
+
+def relu2(z):
+    return np.maximum(z, 0.0) ** 2
+
+
+def zefapel_feed_forward(mlp, W, p, h):
+    if mlp["kind"] == "dense":
+        return (silu(h @ W[p + "gate"].T) * (h @ W[p + "up"].T)) @ W[p + "down"].T
+    r = mlp["router"]
+    E, I = r["experts"], r.get("identity", 0)
+    out = np.zeros_like(h)
+    zs = h @ W[p + "router"].T
+    for t in range(h.shape[0]):
+        for j, w in route(zs[t], W[p + "correction"], r["top"], r["groups"]["count"], r["groups"]["keep"]).items():
+            if j >= E:
+                out[t] += w * h[t]
+            else:
+                out[t] += w * (relu2(h[t] @ W[p + f"e{j}.up"].T) @ W[p + f"e{j}.down"].T)
+    if mlp.get("shared"):
+        shared = relu2(h @ W[p + "shared.up"].T) @ W[p + "shared.down"].T
+        out = out + shared * sigmoid(h @ W[p + "shared.sg"].T)
+    return out
+
+
+def zefapel_forward(config, W, tokens, streams=None):
+    """Logits [L, vocab] of a whole sequence; ``streams`` (a list) receives the residual stream after every layer."""
+    W = {k: np.asarray(v, dtype=np.float64) for k, v in W.items()}
+    eps = config["norm"]["eps"]
+    L = len(tokens)
+    pos = np.arange(L, dtype=np.float64)
+    x = W["embed"][np.asarray(tokens)] * config["embedding"]["scale"]
+    latents = {}
+    for i, spec in enumerate(config["layers"]):
+        p, mc = f"l{i}.", spec["mixer"]
+        h = dyt_norm(x, W[p + "norm1.alpha"], W[p + "norm1"], W[p + "norm1.b"])
+        H, D, V = mc["heads"], mc["dim"], mc["vdim"]
+        m = p + "mix."
+        if spec["type"] == "mlstm":
+            q = (h @ W[m + "q"].T).reshape(L, H, D) * D ** -0.5
+            k = (h @ W[m + "k"].T).reshape(L, H, D)
+            v = (h @ W[m + "v"].T).reshape(L, H, V)
+            cap = mc["gate_cap"]
+            li = cap * np.tanh((h @ W[m + "i"].T + W[m + "i.b"]) / cap)
+            lf = log_sigmoid(cap * np.tanh((h @ W[m + "f"].T + W[m + "f.b"]) / cap))
+            o = rms_norm(matrix_memory(q, k, v, li, lf), None, eps).reshape(L, H * V) * W[m + "norm"]
+            o = o * sigmoid(h @ W[m + "g"].T)
+        elif spec["type"] == "gla":
+            q = (h @ W[m + "q"].T).reshape(L, H, D) * D ** -0.5
+            k = (h @ W[m + "k"].T).reshape(L, H, D)
+            v = (h @ W[m + "v"].T).reshape(L, H, V)
+            z = (h @ W[m + "a1"].T) @ W[m + "a2"].T + W[m + "a2.b"]
+            alpha = np.exp(log_sigmoid(z) / mc["tau"]).reshape(L, H, D)
+            o = rms_norm(gated_linear_attention(q, k, v, alpha), W[m + "norm"], eps).reshape(L, H * V)
+            o = o * silu(h @ W[m + "g"].T)
+        elif spec["type"] == "latent_attention":
+            R, C = mc["rot_dim"], mc["kv_rank"]
+            freqs, mult = scaled_frequencies(mc["rot"]["dims"], mc["rot"]["base"], mc["rot"].get("scaling"))
+            cq = rms_norm(h @ W[m + "dq"].T, W[m + "dq.norm"], eps)
+            q = (cq @ W[m + "uq"].T).reshape(L, H, D + R)
+            q_rot = rotate_pairs_by(q[..., D:], pos, freqs, mult)
+            if "kv_from" in mc:
+                c, k_rot = latents[mc["kv_from"]]
+            else:
+                dkv = h @ W[m + "dkv"].T
+                c = rms_norm(dkv[:, :C], W[m + "dkv.norm"], eps)
+                k_rot = rotate_pairs_by(dkv[:, C:], pos, freqs, mult)
+                latents[i] = (c, k_rot)
+            k_plain = (c @ W[m + "uk"].T).reshape(L, H, D)
+            val = (c @ W[m + "uv"].T).reshape(L, H, V)
+            qq = np.concatenate([q[..., :D], q_rot], -1)
+            kk = np.concatenate([k_plain, np.broadcast_to(k_rot[:, None, :], (L, H, R))], -1)
+            o = causal_softmax_attention(qq, kk, val, mc["scale"]).reshape(L, H * V) * sigmoid(h @ W[m + "g"].T)
+        else:
+            raise ValueError(spec["type"])
+        x = x + W[p + "ls1"] * (o @ W[m + "o"].T)
+        if spec.get("mlp"):
+            h2 = dyt_norm(x, W[p + "norm2.alpha"], W[p + "norm2"], W[p + "norm2.b"])
+            x = x + W[p + "ls2"] * zefapel_feed_forward(spec["mlp"], W, p + "mlp.", h2)
+        if streams is not None:
+            streams.append(x.copy())
+    xf = dyt_norm(x, W["final.norm.alpha"], W["final.norm"], W["final.norm.b"])
+    return xf @ W["head"].T

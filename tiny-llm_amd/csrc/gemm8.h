@@ -32,6 +32,7 @@ struct Gemm8Args {
     int M, N, K;
     float *out_f32 = nullptr;  // EPI_F32_STORE / EPI_F32_AXPY: [M, N] float32 (a float32 residual stream or float32 projections behind bf16 operands)
     float alpha = 1.f;         // EPI_F32_AXPY: out_f32 += alpha * product
+    const float *col_scale = nullptr;  // EPI_F32_AXPY, optional [N]: out_f32 += alpha * col_scale[n] * product (a per-channel scale of the branch)
 };
 // epilogues beside EPI_STORE / EPI_RESIDUAL / EPI_SWIGLU (qmv.h): the accumulators leave as float32
 enum { EPI_F32_STORE = 3, EPI_F32_AXPY = 4 };

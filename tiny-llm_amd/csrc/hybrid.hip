@@ -47,6 +47,8 @@ struct Run {
     bool enters_pass = false; // the loop-entry projection + pass offset come right before this run
     void *kpool = nullptr, *vpool = nullptr;      // attention: [pages, G, page, dim] / [pages, G, page, vdim] of the engine dtype
     float *state = nullptr, *conv_state = nullptr; // delta: [slots, H, vdim, dim] / [slots, taps-1, C]
+                                                   // linrec: [slots, H, vdim (+1), dim] / the gates' running maximum [slots, H]
+    // latent: kpool = [pages, page, kv_rank + rot_dim] (vpool unused); with kv_from the pages of an earlier run (not owned)
 };
 
 struct Meta {  // device int32 arrays of one step
@@ -61,6 +63,9 @@ struct tl_hybrid {
     std::vector<tl_hybrid_layer> layers;
     std::vector<tl::hy::Run> runs;
     std::vector<float *> inv_freq;  // per layer (attention with rotary positions), device
+    std::vector<float> rot_mult;    // per layer: factor on cos and sin (rescaled frequencies)
+    float *f32a = nullptr, *gates = nullptr, *idw = nullptr;  // [R, max_c] scratch (conv output, latent queries, channel decays); [R, H, 3]; [R]
+    void *da = nullptr, *db = nullptr;                         // D-typed scratch rows: latents / low-rank inputs / attention read-out; plain queries
     hipStream_t stream = nullptr;
     bool owns_stream = false;
     std::unique_ptr<tl::PagePool> pool;
@@ -69,7 +74,7 @@ struct tl_hybrid {
     // workspace
     float *part_acc = nullptr, *part_ml = nullptr;  // attention partials of split key ranges: [max_slots, heads, 64, vdim] / [..., 2]
     bool attn_rows_only = false;                    // TL_HYBRID_ATTN_ROWS=1: the one-wave-per-row attention everywhere (A/B twin of the tile kernel)
-    float *x = nullptr, *x0 = nullptr, *proj = nullptr, *qbuf = nullptr, *conv_out = nullptr, *obuf = nullptr, *logits = nullptr;
+    float *x = nullptr, *x0 = nullptr, *proj = nullptr, *qbuf = nullptr, *obuf = nullptr, *logits = nullptr;
     void *h = nullptr, *cat = nullptr, *cat2 = nullptr, *hsel = nullptr;
     int ld_proj = 0, ld_cat = 0;
     int32_t *meta_dev = nullptr, *meta_host = nullptr;  // step metadata (host side pinned)
@@ -93,11 +98,28 @@ namespace hy {
 
 static size_t esize(int dtype) { return dtype == TL_HY_BF16 ? 2 : 4; }
 
-static int in_cols(const tl_hybrid_layer &L) {  // rows of w_in
-    if (L.kind == TL_MIX_ATTENTION) return L.heads * L.dim + L.kv_heads * L.dim + L.kv_heads * L.vdim + (L.gated ? L.heads * L.vdim : 0) + L.ff;
-    return 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim + 2 * L.heads + L.ff;
+static int mixer_cols(const tl_hybrid_layer &L) {  // rows of w_in that belong to the mixer
+    if (L.kind == TL_MIX_ATTENTION) return L.heads * L.dim + L.kv_heads * L.dim + L.kv_heads * L.vdim + (L.gated ? L.heads * L.vdim : 0);
+    if (L.kind == TL_MIX_LINREC) return 2 * L.heads * L.dim + 2 * L.heads * L.vdim + (L.rec_kind == TL_REC_EXPGATE ? 2 * L.heads : L.a_rank);
+    if (L.kind == TL_MIX_LATENT) return L.q_rank + (L.kv_from < 0 ? L.kv_rank + L.rot_dim : 0) + L.heads * L.vdim;
+    return 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim + 2 * L.heads;
+}
+static int ff_in_cols(const tl_hybrid_layer &L) {  // rows of the feed-forward's input matrix
+    if (L.ff <= 0) return 0;
+    if (L.ff_kind == TL_FF_GATED) return 2 * L.ff;
+    if (L.ff_kind == TL_FF_MOE) return L.experts + L.identity + 1 + L.shared_ff + L.experts * L.expert_ff;
+    return L.ff;
 }
 static int conv_channels(const tl_hybrid_layer &L) { return 2 * L.kv_heads * L.dim + L.heads * L.vdim; }
+// floats of one sequence's recurrent state, and of what travels beside it (delta: the convolution's last inputs; expgate: the running maximum)
+static size_t state_floats(const tl_hybrid_layer &L) {
+    if (L.kind == TL_MIX_LINREC) return (size_t)L.heads * L.dim * (L.vdim + (L.rec_kind == TL_REC_EXPGATE ? 1 : 0));
+    return (size_t)L.heads * L.dim * L.vdim;
+}
+static size_t aux_floats(const tl_hybrid_layer &L) {
+    if (L.kind == TL_MIX_LINREC) return (size_t)L.heads;
+    return (size_t)std::max(1, L.conv_taps - 1) * conv_channels(L);
+}
 
 template <typename T>
 static int dev_alloc(tl_hybrid *e, T **p, size_t count, bool zero = false) {
@@ -125,19 +147,21 @@ static size_t meta_ints(int R, int S) { return (size_t)5 * R + 2 * S + 2; }
 // out (+)= A . W^T by shape: a few rows stream the weights once per column (row kernel), more go through the MFMA tile kernel
 template <typename D>
 static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, int M, int N, int K, int epi, float alpha, const float *bias,
-                    int force, hipStream_t st) {
+                    int force, hipStream_t st, int batch = 1, long sa = 0, long sw = 0, long sc = 0) {
     using S = typename D::storage;
-    if (M <= 0 || N <= 0) return TL_OK;
-    const int vec_ok = (K % 8 == 0) && (lda % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+    if (M <= 0 || N <= 0 || batch <= 0) return TL_OK;
+    const int vec_ok = (K % 8 == 0) && (lda % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && sa % 8 == 0 && sw % 8 == 0;
     const bool rows = force == 1 || (force == 0 && M <= 8);
     TL_REQUIRE(!rows || M <= 8, "hybrid linear: the row kernel takes at most 8 rows");
     if constexpr (sizeof(S) == 2) {
         // large bf16 products: the framework's LDS-DMA 256-wide tile GEMM with its float32 epilogues (gemm8.h); dense operands, whole 64-wide K steps
         const bool big = force == 3 || (force == 0 && M >= 192);
-        if (big && lda == K && ldc == N && gemm8_applicable(M, N, K) && (size_t)M * N * 4 < (1ull << 31)) {
+        if (big && batch == 1 && lda == K && ldc == N && gemm8_applicable(M, N, K) && (size_t)M * N * 4 < (1ull << 31) &&
+            (epi != 3 || (uintptr_t)bias % 16 == 0)) {
             Gemm8Args g{};
             g.a = (const uint16_t *)A, g.w = (const uint16_t *)W, g.M = M, g.N = N, g.K = K, g.out_f32 = out, g.alpha = alpha;
-            if (launch_gemm8_bf16(g, epi == 1 ? EPI_F32_AXPY : EPI_F32_STORE, st) == 0) {
+            if (epi == 3) g.col_scale = bias;
+            if (launch_gemm8_bf16(g, (epi == 1 || epi == 3) ? EPI_F32_AXPY : EPI_F32_STORE, st) == 0) {
                 if (epi == 2) {
                     const size_t n = (size_t)M * N;
                     hipLaunchKernelGGL(add_rowvec_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, out, bias, N, M);
@@ -148,17 +172,21 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
         }
         TL_REQUIRE(force != 3, "hybrid linear: the 256-wide tile GEMM does not take this shape");
     }
+#define HY_GEMM(KERN, E) hipLaunchKernelGGL((KERN<D, E>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok, sa, sw, sc)
     if (rows) {
-        dim3 grid((N + 3) / 4), block(256);
-        if (epi == 0) hipLaunchKernelGGL((gemm_rows_kernel<D, 0>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
-        else if (epi == 1) hipLaunchKernelGGL((gemm_rows_kernel<D, 1>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
-        else hipLaunchKernelGGL((gemm_rows_kernel<D, 2>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+        dim3 grid((N + 3) / 4, batch), block(256);
+        if (epi == 0) HY_GEMM(gemm_rows_kernel, 0);
+        else if (epi == 1) HY_GEMM(gemm_rows_kernel, 1);
+        else if (epi == 2) HY_GEMM(gemm_rows_kernel, 2);
+        else HY_GEMM(gemm_rows_kernel, 3);
     } else {
-        dim3 grid(((M + 63) / 64) * ((N + 63) / 64)), block(256);
-        if (epi == 0) hipLaunchKernelGGL((gemm_tile_kernel<D, 0>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
-        else if (epi == 1) hipLaunchKernelGGL((gemm_tile_kernel<D, 1>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
-        else hipLaunchKernelGGL((gemm_tile_kernel<D, 2>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok);
+        dim3 grid(((M + 63) / 64) * ((N + 63) / 64), batch), block(256);
+        if (epi == 0) HY_GEMM(gemm_tile_kernel, 0);
+        else if (epi == 1) HY_GEMM(gemm_tile_kernel, 1);
+        else if (epi == 2) HY_GEMM(gemm_tile_kernel, 2);
+        else HY_GEMM(gemm_tile_kernel, 3);
     }
+#undef HY_GEMM
     TL_CHECK_LAUNCH("hybrid linear");
     return TL_OK;
 }
@@ -177,7 +205,7 @@ static int launch_delta(const tl_hybrid *e, const tl_hybrid_layer &L, const Run 
     const int C = conv_channels(L);
     const int a0 = 2 * L.kv_heads * L.dim + 2 * L.heads * L.vdim, b0 = a0 + L.heads;
 #define HY_DELTA(RPT, LPC)                                                                                                                  \
-    hipLaunchKernelGGL((delta_kernel<RPT, LPC>), grid, block, 0, e->stream, e->conv_out, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
+    hipLaunchKernelGGL((delta_kernel<RPT, LPC>), grid, block, 0, e->stream, e->f32a, C, e->proj, ldp, a0, b0, L.a_log_dev, L.dt_bias_dev, \
                        L.unit_eps, m.seq_row0, m.seq_slot, run.state, e->obuf, L.heads, L.kv_heads, L.dim, L.vdim)
 #define HY_DELTA_R(LPC)                          \
     switch (rpt) {                               \
@@ -227,8 +255,8 @@ static void plan_splits(StepShape &sh, int ctx_bound) {
 }
 
 template <typename D, int DK4, int VT>
-static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, const StepShape &sh, const float *gate, int ldg,
-                            int ldo) {
+static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, int v_row, const Meta &m, const StepShape &sh,
+                            const float *gate, int ldg, void *out, int ldo) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
     const int HG = L.heads / L.kv_heads;
@@ -239,34 +267,202 @@ static int launch_attn_tile(tl_hybrid *e, const tl_hybrid_layer &L, const Run &r
     int page_shift = -1;
     for (int b = 0; b < 30; ++b)
         if ((1 << b) == c.page_size) page_shift = b;
-    const int vec_ok = L.dim % 8 == 0 && L.vdim % 8 == 0;
+    const int vec_ok = L.dim % 8 == 0 && L.vdim % 8 == 0 && v_row % 8 == 0;
     // chunks whose rows fit one 16-row MFMA tile (decode steps): the four waves share the keys of a tile instead of the rows
     const bool wsplit = sh.max_len * HGB <= 16;
     const size_t lds = std::max(lds_tiles, (size_t)(128 + 4 * 64 * 4 * VT) * 4);
     auto kern = wsplit ? attn_tile_kernel<D, DK4, VT, true> : attn_tile_kernel<D, DK4, VT, false>;
     (void)hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     dim3 grid((sh.max_len + TQ - 1) / TQ, L.kv_heads * n_hblk, sh.n_seqs * sh.n_splits);
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)run.kpool, (const S *)run.vpool, m.seq_row0, m.seq_slot, m.row_pos,
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, e->stream, e->qbuf, (const S *)kpool, (const S *)vpool, m.seq_row0, m.seq_slot, m.row_pos,
                        e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim, L.vdim, L.scale, L.sink, HGB, n_hblk, sh.keys_per_split,
-                       sh.n_splits, gate, ldg, (S *)e->cat, ldo, e->part_acc, e->part_ml, page_shift, vec_ok);
+                       sh.n_splits, gate, ldg, (S *)out, ldo, e->part_acc, e->part_ml, page_shift, vec_ok, v_row);
     TL_CHECK_LAUNCH("hybrid attention tile");
     if (sh.n_splits > 1) {
         hipLaunchKernelGGL((attn_merge_kernel<D>), dim3(sh.rows, L.heads), dim3(64), 0, e->stream, e->part_acc, e->part_ml, sh.n_splits, L.heads, L.vdim, gate,
-                           ldg, (S *)e->cat, ldo);
+                           ldg, (S *)out, ldo);
         TL_CHECK_LAUNCH("hybrid attention merge");
     }
+    return TL_OK;
+}
+
+// the attention core over one K/V pool by head widths: the MFMA tile kernel where its templates reach, the row kernel beyond
+template <typename D>
+static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kpool, const void *vpool, int v_row, const Meta &m, const StepShape &sh,
+                          const float *gate, int ldg, void *out, int ldo) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
+    if (e->attn_rows_only || dk4 > 64 || vt_n > 16) {
+        hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(sh.rows, L.heads), dim3(64), (L.dim + 64) * sizeof(float), e->stream, e->qbuf, (const S *)kpool,
+                           (const S *)vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, L.heads, L.kv_heads, L.dim,
+                           L.vdim, L.scale, L.sink, gate, ldg, (S *)out, ldo, v_row);
+        TL_CHECK_LAUNCH("hybrid attention");
+        return TL_OK;
+    }
+    if (dk4 <= 16 && vt_n <= 4) return launch_attn_tile<D, 16, 4>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
+    if (dk4 <= 32 && vt_n <= 8) return launch_attn_tile<D, 32, 8>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
+    return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
+}
+
+static int launch_linrec(const tl_hybrid *e, const tl_hybrid_layer &L, const Run &run, const Meta &m, int n_seqs, int ldp) {
+    const bool chan = L.rec_kind == TL_REC_CHANNEL;
+    const int ones = chan ? 0 : 1, VE = L.vdim + ones;
+    // lanes per state column: a wave while the step's columns are few (decode), a DPP row of 16 otherwise (or for narrow keys)
+    const long cols = (long)L.heads * VE * n_seqs, simds = 4 * (long)qmm3_num_cus();
+    int lpc = (cols <= simds && L.dim > 16) ? 64 : 16;
+    if (L.dim > 16 * 16) lpc = 64;
+    int rpt = 1;
+    while (lpc * rpt < L.dim) rpt *= 2;
+    TL_REQUIRE(rpt <= 16, "hybrid linrec: key width above 1024 is not supported");
+    dim3 grid(L.heads, n_seqs, (VE + 256 / lpc - 1) / (256 / lpc)), block(256);
+    const int q0 = 0, k0 = L.heads * L.dim, v0 = 2 * L.heads * L.dim;
+#define HY_LR(RPT, LPC, CHAN)                                                                                                                      \
+    hipLaunchKernelGGL((linrec_kernel<RPT, LPC, CHAN>), grid, block, 0, e->stream, e->proj, ldp, q0, k0, v0, e->gates, e->f32a, m.seq_row0, m.seq_slot, \
+                       run.state, e->obuf, L.heads, L.dim, L.vdim, ones)
+#define HY_LR_R(LPC, CHAN)                    \
+    switch (rpt) {                            \
+        case 1: HY_LR(1, LPC, CHAN); break;   \
+        case 2: HY_LR(2, LPC, CHAN); break;   \
+        case 4: HY_LR(4, LPC, CHAN); break;   \
+        case 8: HY_LR(8, LPC, CHAN); break;   \
+        default: HY_LR(16, LPC, CHAN); break; \
+    }
+    if (lpc == 64) {
+        if (chan) { HY_LR_R(64, true) } else { HY_LR_R(64, false) }
+    } else {
+        if (chan) { HY_LR_R(16, true) } else { HY_LR_R(16, false) }
+    }
+#undef HY_LR_R
+#undef HY_LR
+    TL_CHECK_LAUNCH("hybrid linrec");
+    return TL_OK;
+}
+
+template <typename D>
+static int norm_t(tl_hybrid *e, int kind, const float *w, const float *b, float alpha, float offset, void *out, const int32_t *rows_idx, int rows) {
+    using S = typename D::storage;
+    const tl_hybrid_config &c = e->cfg;
+    if (kind == TL_NORM_DYT) hipLaunchKernelGGL((dyt_kernel<D>), dim3(rows), dim3(256), 0, e->stream, e->x, w, b, alpha, (S *)out, c.width, rows_idx);
+    else hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(256), 0, e->stream, e->x, w, offset, c.norm_eps, (S *)out, c.width, rows_idx);
+    TL_CHECK_LAUNCH("hybrid norm");
+    return TL_OK;
+}
+
+// the token mixer of one layer run: proj [rows, ldp] (every projection of the normed input) -> cat[:, 0 .. heads * vdim) as D rows of ldcat
+template <typename D>
+static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, int ldp, int ldcat) {
+    using S = typename D::storage;
+    const Run &run = e->runs[ri];
+    const tl_hybrid_layer &L = e->layers[run.layer];
+    const tl_hybrid_config &c = e->cfg;
+    hipStream_t st = e->stream;
+    const int rows = sh.rows, n_seqs = sh.n_seqs, H = L.heads, HV = L.heads * L.vdim;
+    if (L.kind == TL_MIX_ATTENTION) {
+        const int G = L.kv_heads;
+        hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot,
+                           e->table_dev, c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.qk_unit_rms, c.norm_eps, H, G, L.dim,
+                           L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
+        TL_CHECK_LAUNCH("hybrid attention prep");
+        const float *gate = L.gated ? e->proj + (size_t)(H + G) * L.dim + (size_t)G * L.vdim : nullptr;
+        return attention_core<D>(e, L, run.kpool, run.vpool, L.vdim, m, sh, gate, ldp, e->cat, ldcat);
+    }
+    if (L.kind == TL_MIX_LATENT) {
+        // proj: dq (q_rank) | [dkv (kv_rank + rot_dim)] | gate (H * vdim)
+        const int own = L.kv_from < 0, kv0 = L.q_rank, g0 = L.q_rank + (own ? L.kv_rank + L.rot_dim : 0), DT = L.kv_rank + L.rot_dim, DQ = L.dim + L.rot_dim;
+        hipLaunchKernelGGL((rms_cols_kernel<D>), dim3(rows), dim3(64), 0, st, e->proj, ldp, L.q_rank, L.dq_norm_dev, c.norm_eps, (S *)e->da, L.q_rank);
+        TL_CHECK_LAUNCH("hybrid latent query norm");
+        HY_TRY(linear_t<D>(e->da, L.q_rank, L.uq_dev, e->f32a, H * DQ, rows, H * DQ, L.q_rank, 0, 1.f, nullptr, 0, st));
+        hipLaunchKernelGGL((latent_prep_kernel<D>), dim3(rows, H + 1), dim3(64), 0, st, e->f32a, H, L.dim, L.rot_dim, L.kv_rank, e->proj, ldp, kv0,
+                           L.dkv_norm_dev, c.norm_eps, own, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size,
+                           e->inv_freq[run.layer], L.rot_dims, e->rot_mult[run.layer], (S *)e->db, e->qbuf, (S *)run.kpool);
+        TL_CHECK_LAUNCH("hybrid latent prep");
+        // the keys' per-head projection moves onto the query: q_h' = W_uk,h^T q_h  -> qbuf[t, h, 0 .. kv_rank)
+        HY_TRY(linear_t<D>(e->db, H * L.dim, L.uk_t_dev, e->qbuf, H * DT, rows, L.kv_rank, L.dim, 0, 1.f, nullptr, 0, st, H, L.dim, (long)L.kv_rank * L.dim, DT));
+        tl_hybrid_layer A = L;  // one K/V head: keys [c | rotated part], values = the keys' leading kv_rank columns
+        A.kv_heads = 1, A.dim = DT, A.vdim = L.kv_rank, A.sink = 0;
+        HY_TRY(attention_core<D>(e, A, run.kpool, run.kpool, DT, m, sh, nullptr, 0, e->da, H * L.kv_rank));
+        // ... and the values' onto the read-out: o_h = W_uv,h (sum_j p_j c_j)
+        HY_TRY(linear_t<D>(e->da, H * L.kv_rank, L.uv_dev, e->obuf, HV, rows, L.vdim, L.kv_rank, 0, 1.f, nullptr, 0, st, H, L.kv_rank, (long)L.vdim * L.kv_rank, L.vdim));
+        const size_t n = (size_t)rows * HV;
+        hipLaunchKernelGGL((gate_mul_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->obuf, HV, e->proj + g0, ldp, HV, 0, (S *)e->cat, ldcat, rows);
+        TL_CHECK_LAUNCH("hybrid latent gate");
+        return TL_OK;
+    }
+    if (L.kind == TL_MIX_LINREC) {
+        // proj: q (H dim) | k (H dim) | v (H vdim) | gate (H vdim) | i (H) | f (H)   or   ... | a1 (a_rank)
+        const int g0 = 2 * H * L.dim + HV, x0 = g0 + HV;
+        const bool chan = L.rec_kind == TL_REC_CHANNEL;
+        if (chan) {
+            const size_t na = (size_t)rows * L.a_rank, nd = (size_t)rows * H * L.dim;
+            hipLaunchKernelGGL((cast_cols_kernel<D>), dim3((unsigned)((na + 255) / 256)), dim3(256), 0, st, e->proj, ldp, x0, L.a_rank, (S *)e->da, L.a_rank, rows);
+            TL_CHECK_LAUNCH("hybrid decay input");
+            HY_TRY(linear_t<D>(e->da, L.a_rank, L.a2_dev, e->f32a, H * L.dim, rows, H * L.dim, L.a_rank, 0, 1.f, nullptr, 0, st));
+            hipLaunchKernelGGL(channel_decay_kernel, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, st, e->f32a, L.a2_bias_dev, H * L.dim, 1.f / L.tau, rows);
+            TL_CHECK_LAUNCH("hybrid channel decay");
+        } else {
+            hipLaunchKernelGGL(expgate_scan_kernel, dim3(n_seqs, H), dim3(64), 0, st, e->proj, ldp, x0, x0 + H, L.i_bias_dev, L.f_bias_dev, L.gate_cap,
+                               m.seq_row0, m.seq_slot, run.conv_state, e->gates, H);
+            TL_CHECK_LAUNCH("hybrid gate scan");
+        }
+        HY_TRY(launch_linrec(e, L, run, m, n_seqs, ldp));
+        hipLaunchKernelGGL((linrec_out_kernel<D>), dim3(rows, H), dim3(64), 0, st, e->obuf, L.vdim + (chan ? 0 : 1), chan ? 0 : 1, e->gates,
+                           1.f / sqrtf((float)L.dim), L.out_norm_dev, chan ? 0 : L.vdim, c.norm_eps, e->proj + g0, ldp, chan ? 1 : 0, H, L.vdim, (S *)e->cat,
+                           ldcat);
+        TL_CHECK_LAUNCH("hybrid linrec out");
+        return TL_OK;
+    }
+    const int C = conv_channels(L);
+    const size_t n = (size_t)rows * C;
+    hipLaunchKernelGGL(conv_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, L.conv_dev, L.conv_taps, C, m.row_seq,
+                       m.seq_row0, m.seq_slot, run.conv_state, e->f32a, rows);
+    TL_CHECK_LAUNCH("hybrid conv");
+    if (L.conv_taps > 1) {
+        hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)(((size_t)n_seqs * C + 255) / 256)), dim3(256), 0, st, e->proj, ldp, L.conv_taps, C,
+                           m.seq_row0, m.seq_slot, run.conv_state, n_seqs);
+        TL_CHECK_LAUNCH("hybrid conv state");
+    }
+    HY_TRY(launch_delta(e, L, run, m, n_seqs, ldp));
+    const float *gate = e->proj + (size_t)C;
+    hipLaunchKernelGGL((delta_out_kernel<D>), dim3(rows, L.heads), dim3(64), 0, st, e->obuf, L.out_norm_dev, c.norm_eps, gate, ldp, L.heads,
+                       L.vdim, (S *)e->cat, ldcat);
+    TL_CHECK_LAUNCH("hybrid delta out");
+    return TL_OK;
+}
+
+// the feed-forward's activation: proj columns up0 .. -> cat columns col0 .. col0 + L.ff
+template <typename D>
+static int ff_act_t(tl_hybrid *e, const tl_hybrid_layer &L, int rows, int ldp, int up0, int ldcat, int col0) {
+    using S = typename D::storage;
+    hipStream_t st = e->stream;
+    if (L.ff_kind == TL_FF_MOE) {
+        const int ET = L.experts + L.identity;
+        hipLaunchKernelGGL((moe_route_act_kernel<D>), dim3(rows), dim3(256), 0, st, e->proj, ldp, up0, up0 + ET, up0 + ET + 1, up0 + ET + 1 + L.shared_ff,
+                           L.experts, L.identity, L.top, L.groups, L.keep, L.expert_ff, L.shared_ff, L.correction_dev, (S *)e->cat, ldcat, col0, e->idw);
+        TL_CHECK_LAUNCH("hybrid moe route");
+        return TL_OK;
+    }
+    const size_t n = (size_t)rows * L.ff;
+    if (L.ff_kind == TL_FF_GATED)
+        hipLaunchKernelGGL((ff_gated_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, up0, up0 + L.ff, L.ff, L.ff_act,
+                           (S *)e->cat, ldcat, col0, rows);
+    else
+        hipLaunchKernelGGL((ff_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, up0, L.ff, L.ff_act, (S *)e->cat, ldcat, col0,
+                           rows);
+    TL_CHECK_LAUNCH("hybrid ff act");
     return TL_OK;
 }
 
 // every layer run over the packed rows described by m
 template <typename D>
 static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
-    const int rows = sh.rows, n_seqs = sh.n_seqs;
+    const int rows = sh.rows;
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
     hipStream_t st = e->stream;
     const int W = c.width;
-    hipLaunchKernelGGL((embed_kernel<D>), dim3(rows), dim3(256), 0, st, m.tokens, (const S *)c.embed_dev, e->x0, e->x, W, c.vocab);
+    hipLaunchKernelGGL((embed_kernel<D>), dim3(rows), dim3(256), 0, st, m.tokens, (const S *)c.embed_dev, e->x0, e->x, W, c.vocab,
+                       c.embed_scale != 0.f ? c.embed_scale : 1.f);
     TL_CHECK_LAUNCH("hybrid embed");
     for (size_t ri = 0; ri < e->runs.size(); ++ri) {
         const Run &run = e->runs[ri];
@@ -276,56 +472,34 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
             TL_CHECK_LAUNCH("hybrid pack2");
             HY_TRY(linear_t<D>(e->cat2, 2 * W, c.loop_in_dev, e->x, W, rows, W, 2 * W, 2, 1.f, c.loop_step_dev + (size_t)run.pass * W, 0, st));
         }
-        hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(256), 0, st, e->x, L.norm_dev, L.norm_offset, c.norm_eps, (S *)e->h, W, (const int32_t *)nullptr);
-        TL_CHECK_LAUNCH("hybrid norm");
-        const int nin = in_cols(L), HV = L.heads * L.vdim;
-        const int ldp = nin, ldcat = HV + L.ff;  // dense rows: a layer's buffers are as wide as the layer needs
-        HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, ldp, rows, nin, W, 0, 1.f, nullptr, 0, st));
-        if (L.kind == TL_MIX_ATTENTION) {
-            const int H = L.heads, G = L.kv_heads;
-            hipLaunchKernelGGL((attn_prep_kernel<D>), dim3(rows, H + 2 * G), dim3(64), 0, st, e->proj, ldp, m.row_seq, m.row_pos, m.seq_slot,
-                               e->table_dev, c.max_pages_per_seq, c.page_size, e->inv_freq[run.layer], L.rot_dims, L.qk_unit_rms, c.norm_eps, H, G, L.dim,
-                               L.vdim, e->qbuf, (S *)run.kpool, (S *)run.vpool);
-            TL_CHECK_LAUNCH("hybrid attention prep");
-            const float *gate = L.gated ? e->proj + (size_t)(H + G) * L.dim + (size_t)G * L.vdim : nullptr;
-            const int dk4 = (L.dim + 3) / 4, vt_n = (L.vdim + 15) / 16;
-            if (e->attn_rows_only || dk4 > 64 || vt_n > 16) {
-                hipLaunchKernelGGL((attn_rows_kernel<D>), dim3(rows, H), dim3(64), (L.dim + 64) * sizeof(float), st, e->qbuf, (const S *)run.kpool,
-                                   (const S *)run.vpool, m.row_seq, m.row_pos, m.seq_slot, e->table_dev, c.max_pages_per_seq, c.page_size, H, G, L.dim, L.vdim,
-                                   L.scale, L.sink, gate, ldp, (S *)e->cat, ldcat);
-                TL_CHECK_LAUNCH("hybrid attention");
-            } else if (dk4 <= 16 && vt_n <= 4) {
-                HY_TRY((launch_attn_tile<D, 16, 4>(e, L, run, m, sh, gate, ldp, ldcat)));
-            } else if (dk4 <= 32 && vt_n <= 8) {
-                HY_TRY((launch_attn_tile<D, 32, 8>(e, L, run, m, sh, gate, ldp, ldcat)));
-            } else {
-                HY_TRY((launch_attn_tile<D, 64, 16>(e, L, run, m, sh, gate, ldp, ldcat)));
-            }
+        HY_TRY(norm_t<D>(e, L.norm_kind, L.norm_dev, L.norm_bias_dev, L.norm_alpha, L.norm_offset, e->h, nullptr, rows));
+        const int nmix = mixer_cols(L), HV = L.heads * L.vdim;
+        if (c.parallel_block) {
+            const int nin = nmix + L.ff, ldcat = HV + L.ff;  // dense rows: a layer's buffers are as wide as the layer needs
+            HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nin, rows, nin, W, 0, 1.f, nullptr, 0, st));
+            HY_TRY(mixer_t<D>(e, ri, m, sh, nin, ldcat));
+            if (L.ff > 0) HY_TRY(ff_act_t<D>(e, L, rows, nin, nmix, ldcat, HV));
+            // x += m * ([mixer out ; ff act] . [W_o | W_down]^T)
+            HY_TRY(linear_t<D>(e->cat, ldcat, L.w_out_dev, e->x, W, rows, W, HV + L.ff, 1, c.residual_mult, nullptr, 0, st));
         } else {
-            const int C = conv_channels(L);
-            const size_t n = (size_t)rows * C;
-            hipLaunchKernelGGL(conv_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, L.conv_dev, L.conv_taps, C, m.row_seq,
-                               m.seq_row0, m.seq_slot, run.conv_state, e->conv_out, rows);
-            TL_CHECK_LAUNCH("hybrid conv");
-            if (L.conv_taps > 1) {
-                hipLaunchKernelGGL(conv_state_kernel, dim3((unsigned)(((size_t)n_seqs * C + 255) / 256)), dim3(256), 0, st, e->proj, ldp, L.conv_taps, C,
-                                   m.seq_row0, m.seq_slot, run.conv_state, n_seqs);
-                TL_CHECK_LAUNCH("hybrid conv state");
+            // x += m ls1 * W_o mixer(norm1 x);  x += m ls2 * ff(norm2 x)
+            HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nmix, rows, nmix, W, 0, 1.f, nullptr, 0, st));
+            HY_TRY(mixer_t<D>(e, ri, m, sh, nmix, HV));
+            HY_TRY(linear_t<D>(e->cat, HV, L.w_out_dev, e->x, W, rows, W, HV, L.ls1_dev ? 3 : 1, c.residual_mult, L.ls1_dev, 0, st));
+            if (L.ff > 0) {
+                HY_TRY(norm_t<D>(e, L.norm_kind, L.norm2_dev, L.norm2_bias_dev, L.norm2_alpha, L.norm_offset, e->h, nullptr, rows));
+                const int nin2 = ff_in_cols(L);
+                HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, nin2, W, 0, 1.f, nullptr, 0, st));
+                HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
+                HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->x, W, rows, W, L.ff, L.ls2_dev ? 3 : 1, c.residual_mult, L.ls2_dev, 0, st));
+                if (L.ff_kind == TL_FF_MOE && L.identity > 0) {
+                    const size_t n = (size_t)rows * W;
+                    hipLaunchKernelGGL((identity_axpy_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->x, (const S *)e->h, e->idw, L.ls2_dev,
+                                       c.residual_mult, W, rows);
+                    TL_CHECK_LAUNCH("hybrid identity experts");
+                }
             }
-            HY_TRY(launch_delta(e, L, run, m, n_seqs, ldp));
-            const float *gate = e->proj + (size_t)C;
-            hipLaunchKernelGGL((delta_out_kernel<D>), dim3(rows, L.heads), dim3(64), 0, st, e->obuf, L.out_norm_dev, c.norm_eps, gate, ldp, L.heads,
-                               L.vdim, (S *)e->cat, ldcat);
-            TL_CHECK_LAUNCH("hybrid delta out");
         }
-        if (L.ff > 0) {
-            const size_t n = (size_t)rows * L.ff;
-            hipLaunchKernelGGL((ff_act_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->proj, ldp, nin - L.ff, L.ff, L.ff_act,
-                               (S *)e->cat, ldcat, HV, rows);
-            TL_CHECK_LAUNCH("hybrid ff act");
-        }
-        // x += m * ([mixer out ; ff act] . [W_o | W_down]^T)
-        HY_TRY(linear_t<D>(e->cat, ldcat, L.w_out_dev, e->x, W, rows, W, HV + L.ff, 1, c.residual_mult, nullptr, 0, st));
         if (e->trace && e->trace_buf && rows <= c.max_rows)
             HY_HIP(hipMemcpyAsync(e->trace_buf + ri * (size_t)c.max_rows * W, e->x, (size_t)rows * W * 4, hipMemcpyDeviceToDevice, st));
     }
@@ -338,9 +512,7 @@ static int head_t(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
     if (n_want <= 0) return TL_OK;
-    hipLaunchKernelGGL((norm_kernel<D>), dim3(n_want), dim3(256), 0, e->stream, e->x, c.final_norm_dev, c.final_norm_offset, c.norm_eps, (S *)e->hsel, c.width,
-                       (const int32_t *)m.want_rows);
-    TL_CHECK_LAUNCH("hybrid final norm");
+    HY_TRY(norm_t<D>(e, c.final_norm_kind, c.final_norm_dev, c.final_norm_bias_dev, c.final_norm_alpha, c.final_norm_offset, e->hsel, m.want_rows, n_want));
     HY_TRY(linear_t<D>(e->hsel, c.width, c.head_dev, e->logits, c.vocab, n_want, c.vocab, c.width, 0, 1.f, nullptr, 0, e->stream));
     hipLaunchKernelGGL(argmax_kernel, dim3(n_want), dim3(1024), 0, e->stream, e->logits, c.vocab, e->argmax_dev, set_pending ? m.want_slot : (const int32_t *)nullptr,
                        e->pending_dev);
@@ -405,7 +577,8 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     const tl_hybrid_config &c = *cfg;
     TL_REQUIRE(c.dtype == TL_HY_BF16 || c.dtype == TL_HY_F32, "hybrid_create: dtype must be bfloat16 or float32");
     TL_REQUIRE(c.width > 0 && c.vocab > 0 && c.num_layers > 0, "hybrid_create: width, vocab and num_layers must be positive");
-    TL_REQUIRE(c.parallel_block == 1, "hybrid_create: only the parallel block (one norm, mixer + feed-forward) is implemented");
+    TL_REQUIRE(c.parallel_block == 0 || c.parallel_block == 1, "hybrid_create: parallel_block is 0 (sequential) or 1 (parallel)");
+    TL_REQUIRE(c.final_norm_kind == TL_NORM_RMS || (c.final_norm_kind == TL_NORM_DYT && c.final_norm_bias_dev), "hybrid_create: final norm kind");
     TL_REQUIRE(c.page_size > 0 && c.num_pages > 0 && c.max_slots > 0 && c.max_pages_per_seq > 0 && c.max_rows > 0, "hybrid_create: pool sizes must be positive");
     TL_REQUIRE(c.embed_dev && c.final_norm_dev && c.head_dev, "hybrid_create: embed, final norm and head are required");
     const bool looped = c.loop_times > 1 || (c.loop_times == 1 && c.loop_stop > c.loop_start);
@@ -422,24 +595,68 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
         HY_HIP(hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking));
         e->owns_stream = true;
     }
-    int max_in = 0, max_cat = 0, max_q = 0, max_c = 0, max_hv = 0;
+    int max_in = 0, max_cat = 0, max_q = 0, max_c = 0, max_hv = 0, max_gh = 1, max_da = 1, max_db = 1;
     for (int i = 0; i < c.num_layers; ++i) {
         const tl_hybrid_layer &L = e->layers[i];
-        TL_REQUIRE(L.kind == TL_MIX_ATTENTION || L.kind == TL_MIX_DELTA, "hybrid_create: unknown mixer kind");
+        TL_REQUIRE(L.kind == TL_MIX_ATTENTION || L.kind == TL_MIX_DELTA || L.kind == TL_MIX_LINREC || L.kind == TL_MIX_LATENT, "hybrid_create: unknown mixer kind");
         TL_REQUIRE(L.heads > 0 && L.kv_heads > 0 && L.heads % L.kv_heads == 0, "hybrid_create: heads must be a positive multiple of kv_heads");
         TL_REQUIRE(L.dim > 0 && L.dim <= 1024 && L.vdim > 0 && L.vdim <= 512, "hybrid_create: head widths: dim 1..1024, vdim 1..512");
         TL_REQUIRE(L.w_in_dev && L.w_out_dev && L.norm_dev && L.ff >= 0, "hybrid_create: layer matrices and norm are required");
+        TL_REQUIRE(L.norm_kind == TL_NORM_RMS || (L.norm_kind == TL_NORM_DYT && L.norm_bias_dev), "hybrid_create: norm kind (Dynamic Tanh needs its bias)");
+        if (c.parallel_block) {
+            TL_REQUIRE(L.ff_kind == TL_FF_PLAIN && !L.ls1_dev && !L.ls2_dev, "hybrid_create: the parallel block takes a plain feed-forward and no layer scale");
+        } else if (L.ff > 0) {
+            TL_REQUIRE(L.norm2_dev && L.w_in2_dev && L.w_out2_dev && (L.norm_kind != TL_NORM_DYT || L.norm2_bias_dev),
+                       "hybrid_create: a sequential block's feed-forward needs its norm and matrices");
+            TL_REQUIRE(L.ff_kind == TL_FF_PLAIN || L.ff_kind == TL_FF_GATED || L.ff_kind == TL_FF_MOE, "hybrid_create: unknown feed-forward kind");
+            if (L.ff_kind == TL_FF_MOE) {
+                const int ET = L.experts + L.identity;
+                TL_REQUIRE(L.experts >= 0 && L.identity >= 0 && ET >= 1 && ET <= 256, "hybrid_create: between 1 and 256 experts (identity experts included)");
+                TL_REQUIRE(L.groups >= 1 && ET % L.groups == 0 && L.keep >= 1 && L.keep <= L.groups, "hybrid_create: expert groups must divide the experts; 1 <= keep <= groups");
+                TL_REQUIRE(L.top >= 1 && L.top <= L.keep * (ET / L.groups), "hybrid_create: top exceeds the experts of the kept groups");
+                TL_REQUIRE(L.expert_ff >= 0 && L.shared_ff >= 0 && L.ff == L.shared_ff + L.experts * L.expert_ff && L.correction_dev,
+                           "hybrid_create: mixture of experts: ff = shared_ff + experts * expert_ff, correction required");
+            }
+        }
         if (L.kind == TL_MIX_ATTENTION) {
             TL_REQUIRE(L.rot_dims >= 0 && L.rot_dims % 2 == 0 && L.rot_dims <= L.dim, "hybrid_create: rot_dims must be even and at most dim");
+        } else if (L.kind == TL_MIX_LINREC) {
+            TL_REQUIRE(L.kv_heads == L.heads && L.out_norm_dev, "hybrid_create: a linear recurrence has one key head per head and an output norm weight");
+            if (L.rec_kind == TL_REC_CHANNEL)
+                TL_REQUIRE(L.a_rank >= 1 && L.a2_dev && L.a2_bias_dev && L.tau > 0.f, "hybrid_create: channel decay needs its projection pair, bias and tau > 0");
+            else
+                TL_REQUIRE(L.rec_kind == TL_REC_EXPGATE && L.i_bias_dev && L.f_bias_dev && L.gate_cap > 0.f, "hybrid_create: exponential gates need biases and a cap > 0");
+        } else if (L.kind == TL_MIX_LATENT) {
+            TL_REQUIRE(L.q_rank >= 1 && L.kv_rank >= 1 && L.rot_dim >= 0 && L.dq_norm_dev && L.uq_dev && L.uk_t_dev && L.uv_dev,
+                       "hybrid_create: latent attention needs its ranks and per-head projections");
+            TL_REQUIRE(L.rot_dims >= 0 && L.rot_dims % 2 == 0 && L.rot_dims <= L.rot_dim, "hybrid_create: rot_dims must be even and at most rot_dim");
+            TL_REQUIRE(L.kv_rank + L.rot_dim <= 1024 && L.kv_rank <= 512, "hybrid_create: latent widths: kv_rank + rot_dim <= 1024, kv_rank <= 512");
+            if (L.kv_from >= 0) {
+                TL_REQUIRE(L.kv_from < i, "hybrid_create: kv_from must name an earlier layer");
+                const tl_hybrid_layer &J = e->layers[L.kv_from];
+                TL_REQUIRE(J.kind == TL_MIX_LATENT && J.kv_from < 0 && J.kv_rank == L.kv_rank && J.rot_dim == L.rot_dim,
+                           "hybrid_create: kv_from must name a latent-attention layer with its own latent of the same widths");
+            } else {
+                TL_REQUIRE(L.dkv_norm_dev, "hybrid_create: a latent of its own needs its norm weight");
+            }
         } else {
             TL_REQUIRE(L.conv_taps >= 1 && L.conv_taps <= 64 && L.conv_dev && L.a_log_dev && L.dt_bias_dev && L.out_norm_dev,
                        "hybrid_create: a delta layer needs conv taps and weights, a_log, dt_bias and its output norm");
         }
-        max_in = std::max(max_in, in_cols(L));
-        max_cat = std::max(max_cat, L.heads * L.vdim + L.ff);
-        max_hv = std::max(max_hv, L.heads * L.vdim);
+        max_in = std::max(max_in, c.parallel_block ? mixer_cols(L) + L.ff : std::max(mixer_cols(L), ff_in_cols(L)));
+        max_cat = std::max(max_cat, c.parallel_block ? L.heads * L.vdim + L.ff : std::max(L.heads * L.vdim, L.ff));
+        max_hv = std::max(max_hv, L.heads * (L.vdim + 1));
+        max_gh = std::max(max_gh, L.heads);
         if (L.kind == TL_MIX_ATTENTION) max_q = std::max(max_q, L.heads * L.dim);
-        else max_c = std::max(max_c, conv_channels(L));
+        else if (L.kind == TL_MIX_LATENT) {
+            max_q = std::max(max_q, L.heads * (L.kv_rank + L.rot_dim));
+            max_c = std::max(max_c, L.heads * (L.dim + L.rot_dim));
+            max_da = std::max(max_da, std::max(L.q_rank, L.heads * L.kv_rank));
+            max_db = std::max(max_db, L.heads * L.dim);
+        } else if (L.kind == TL_MIX_LINREC) {
+            max_c = std::max(max_c, L.heads * L.dim);
+            max_da = std::max(max_da, L.a_rank);
+        } else max_c = std::max(max_c, conv_channels(L));
     }
     // layer runs
     for (int i = 0; i < c.num_layers;) {
@@ -462,18 +679,51 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     tl_hybrid *p = e.get();
     const size_t es = esize(c.dtype);
     e->inv_freq.assign(c.num_layers, nullptr);
+    e->rot_mult.assign(c.num_layers, 1.f);
     for (int i = 0; i < c.num_layers; ++i) {
         const tl_hybrid_layer &L = e->layers[i];
-        if (L.kind != TL_MIX_ATTENTION) continue;
+        if (L.kind != TL_MIX_ATTENTION && L.kind != TL_MIX_LATENT) continue;
         const int half = std::max(1, L.rot_dims / 2);
         std::vector<float> f(half, 0.f);
         for (int k = 0; k < L.rot_dims / 2; ++k) f[k] = (float)std::pow((double)L.rot_base, -2.0 * k / (double)L.rot_dims);
+        if (L.rot_factor > 0.f && L.rot_dims > 0) {
+            // rescaled frequencies: where(t) = the dimension that turns t times over `original` positions; dimensions below where(fast) keep
+            // their frequency, those above where(slow) are slowed by `factor`, a linear ramp between; cos and sin grow by 0.1 ln(factor) + 1
+            const double two_pi = 6.283185307179586476925287, dims = L.rot_dims, lb = std::log((double)L.rot_base);
+            auto where = [&](double turns) { return dims * std::log((double)L.rot_original / (two_pi * turns)) / (2.0 * lb); };
+            const double lo = std::max(std::floor(where(L.rot_fast)), 0.0), hi = std::min(std::ceil(where(L.rot_slow)), dims - 1.0);
+            for (int k = 0; k < L.rot_dims / 2; ++k) {
+                const double fk = std::pow((double)L.rot_base, -2.0 * k / dims);
+                const double ramp = std::min(1.0, std::max(0.0, (k - lo) / std::max(hi - lo, 0.001)));
+                f[k] = (float)(fk / (double)L.rot_factor * ramp + fk * (1.0 - ramp));
+            }
+            e->rot_mult[i] = (float)(0.1 * std::log((double)L.rot_factor) + 1.0);
+        }
         HY_TRY(dev_alloc(p, &e->inv_freq[i], half));
         HY_HIP(hipMemcpy(e->inv_freq[i], f.data(), half * 4, hipMemcpyHostToDevice));
     }
-    for (Run &r : e->runs) {
+    for (size_t ri = 0; ri < e->runs.size(); ++ri) {
+        Run &r = e->runs[ri];
         const tl_hybrid_layer &L = e->layers[r.layer];
-        if (L.kind == TL_MIX_ATTENTION) {
+        if (L.kind == TL_MIX_LATENT) {
+            if (L.kv_from >= 0) {  // the pages of the latest earlier run of that layer (the same loop pass, or the last pass before)
+                for (size_t rj = ri; rj-- > 0;)
+                    if (e->runs[rj].layer == L.kv_from) {
+                        r.kpool = e->runs[rj].kpool;
+                        break;
+                    }
+                TL_REQUIRE(r.kpool, "hybrid_create: kv_from names a layer that has not run before this one");
+            } else {
+                const size_t kb = (size_t)c.num_pages * c.page_size * (L.kv_rank + L.rot_dim) * es;
+                HY_TRY(dev_alloc(p, (char **)&r.kpool, kb, true));
+                e->stats.kv_bytes += kb;
+            }
+        } else if (L.kind == TL_MIX_LINREC) {
+            const size_t sb = (size_t)c.max_slots * L.heads * L.dim * (L.vdim + (L.rec_kind == TL_REC_EXPGATE ? 1 : 0)), mb = (size_t)c.max_slots * L.heads;
+            HY_TRY(dev_alloc(p, &r.state, sb, true));
+            HY_TRY(dev_alloc(p, &r.conv_state, mb, true));
+            e->stats.state_bytes += (sb + mb) * 4;
+        } else if (L.kind == TL_MIX_ATTENTION) {
             const size_t kb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.dim * es, vb = (size_t)c.num_pages * L.kv_heads * c.page_size * L.vdim * es;
             HY_TRY(dev_alloc(p, (char **)&r.kpool, kb, true));
             HY_TRY(dev_alloc(p, (char **)&r.vpool, vb, true));
@@ -493,12 +743,17 @@ extern "C" int tl_hybrid_create(const tl_hybrid_config *cfg, const tl_hybrid_lay
     HY_TRY(dev_alloc(p, &e->x0, (size_t)R * W));
     HY_TRY(dev_alloc(p, &e->proj, (size_t)R * e->ld_proj));
     HY_TRY(dev_alloc(p, &e->qbuf, (size_t)R * std::max(1, max_q)));
-    HY_TRY(dev_alloc(p, &e->conv_out, (size_t)R * std::max(1, max_c)));
+    HY_TRY(dev_alloc(p, &e->f32a, (size_t)R * std::max(1, max_c)));
+    HY_TRY(dev_alloc(p, &e->gates, (size_t)R * max_gh * 3));
+    HY_TRY(dev_alloc(p, &e->idw, (size_t)R));
+    HY_TRY(dev_alloc(p, (char **)&e->da, (size_t)R * max_da * es));
+    HY_TRY(dev_alloc(p, (char **)&e->db, (size_t)R * max_db * es));
     HY_TRY(dev_alloc(p, &e->obuf, (size_t)R * std::max(1, max_hv)));
     HY_TRY(dev_alloc(p, &e->logits, (size_t)R * c.vocab));
     int max_h = 1, max_v = 1;
     for (const tl_hybrid_layer &L : e->layers)
         if (L.kind == TL_MIX_ATTENTION) max_h = std::max(max_h, L.heads), max_v = std::max(max_v, L.vdim);
+        else if (L.kind == TL_MIX_LATENT) max_h = std::max(max_h, L.heads), max_v = std::max(max_v, L.kv_rank);
     HY_TRY(dev_alloc(p, &e->part_acc, (size_t)c.max_slots * max_h * 64 * max_v));
     HY_TRY(dev_alloc(p, &e->part_ml, (size_t)c.max_slots * max_h * 64 * 2));
     if (const char *v = getenv("TL_HYBRID_ATTN_ROWS")) e->attn_rows_only = v[0] != '\0' && v[0] != '0';
@@ -547,8 +802,8 @@ extern "C" int tl_hybrid_begin(tl_hybrid *e, int slot) {
     e->pool->begin(slot);
     for (Run &r : e->runs) {  // the slot's recurrent state starts at zero (fill kernels: a caller may have a capture open on this stream)
         const tl_hybrid_layer &L = e->layers[r.layer];
-        if (L.kind != TL_MIX_DELTA) continue;
-        const size_t sn = (size_t)L.heads * L.dim * L.vdim, cn = (size_t)std::max(1, L.conv_taps - 1) * conv_channels(L);
+        if (L.kind != TL_MIX_DELTA && L.kind != TL_MIX_LINREC) continue;
+        const size_t sn = state_floats(L), cn = aux_floats(L);
         hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<size_t>(1024, (sn + 255) / 256)), dim3(256), 0, e->stream, r.state + slot * sn, sn, 0.f);
         hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<size_t>(1024, (cn + 255) / 256)), dim3(256), 0, e->stream, r.conv_state + slot * cn, cn, 0.f);
         TL_CHECK_LAUNCH("hybrid_begin: state fill");
@@ -571,8 +826,8 @@ extern "C" int tl_hybrid_move(tl_hybrid *e, int src, int dst) {
     TL_REQUIRE(e->pool->live(src) && !e->pool->live(dst), "hybrid_move: src must hold a sequence and dst must be free");
     for (Run &r : e->runs) {  // recurrent state and convolution inputs travel with the sequence; K/V pages stay where they are
         const tl_hybrid_layer &L = e->layers[r.layer];
-        if (L.kind != TL_MIX_DELTA) continue;
-        const size_t sn = (size_t)L.heads * L.dim * L.vdim, cn = (size_t)std::max(1, L.conv_taps - 1) * conv_channels(L);
+        if (L.kind != TL_MIX_DELTA && L.kind != TL_MIX_LINREC) continue;
+        const size_t sn = state_floats(L), cn = aux_floats(L);
         HY_HIP(hipMemcpyAsync(r.state + dst * sn, r.state + src * sn, sn * 4, hipMemcpyDeviceToDevice, e->stream));
         HY_HIP(hipMemcpyAsync(r.conv_state + dst * cn, r.conv_state + src * cn, cn * 4, hipMemcpyDeviceToDevice, e->stream));
     }

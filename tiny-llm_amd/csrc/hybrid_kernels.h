@@ -34,14 +34,14 @@ __device__ __forceinline__ float act_f(float z, int kind) {
     return silu_f(z);
 }
 
-// ---- embedding gather: x0 = x = embed[token] -------------------------------------------------------------------
+// ---- embedding gather: x0 = x = embed[token] * scale -----------------------------------------------------------
 template <typename D>
-__global__ void embed_kernel(const int32_t *tokens, const typename D::storage *embed, float *x0, float *x, int width, int vocab) {
+__global__ void embed_kernel(const int32_t *tokens, const typename D::storage *embed, float *x0, float *x, int width, int vocab, float scale) {
     const int t = blockIdx.x;
     int tok = tokens[t];
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
     for (int c = threadIdx.x; c < width; c += blockDim.x) {
-        const float v = ld<D>(embed, (size_t)tok * width + c);
+        const float v = ld<D>(embed, (size_t)tok * width + c) * scale;
         x0[(size_t)t * width + c] = v;
         x[(size_t)t * width + c] = v;
     }
@@ -72,11 +72,14 @@ __global__ void pack2_kernel(const float *x, const float *x0, typename D::storag
 // ---- tile matrix product: out[M, N] (+)= A[M, K] . W[N, K]^T, float32 accumulation on the matrix cores ------------
 // 64 x 64 output tile per 256-thread workgroup, 4 waves of 32 x 32 (2 x 2 MFMA 16x16 tiles), K in steps of 32 through LDS.
 // bf16: v_mfma_f32_16x16x32_bf16; fp32: v_mfma_f32_16x16x4_f32 (full fp32 products).  Any M, N, K: edges are zero-filled in LDS.
-// EPI 0: out = acc   1: out += alpha * acc   2: out = acc + bias[n]
+// EPI 0: out = acc   1: out += alpha * acc   2: out = acc + bias[n]   3: out += alpha * bias[n] * acc (a per-column scale on the way into the sum)
+// blockIdx.y = a batch of independent products of one shape (the heads of a per-head projection): operands advance by sa / sw / sc elements.
 template <typename D, int EPI>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
-                                                        int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok) {
+                                                        int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok, long sa, long sw,
+                                                        long sc) {
     using S = typename D::storage;
+    A += (size_t)blockIdx.y * sa, W += (size_t)blockIdx.y * sw, out += (size_t)blockIdx.y * sc;
     constexpr bool BF = sizeof(S) == 2;
     constexpr int KT = 32, LD = BF ? KT + 8 : KT + 1;
     __shared__ S As[64 * LD];
@@ -173,7 +176,8 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storag
                     const float v = acc[i][j][r];
                     if constexpr (EPI == 0) *o = v;
                     else if constexpr (EPI == 1) *o += alpha * v;
-                    else *o = v + bias[gn];
+                    else if constexpr (EPI == 2) *o = v + bias[gn];
+                    else *o += alpha * bias[gn] * v;
                 }
             }
 }
@@ -182,8 +186,10 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storag
 // M <= 8.  Lanes stride over K, 8 elements at a time where the layout allows 16-byte loads.
 template <typename D, int EPI>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
-                                                        int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok) {
+                                                        int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok, long sa, long sw,
+                                                        long sc) {
     using S = typename D::storage;
+    A += (size_t)blockIdx.y * sa, W += (size_t)blockIdx.y * sw, out += (size_t)blockIdx.y * sc;
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N) return;
@@ -236,7 +242,8 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const typename D::storag
                 float *o = out + (size_t)m * ldc + n;
                 if constexpr (EPI == 0) *o = v;
                 else if constexpr (EPI == 1) *o += alpha * v;
-                else *o = v + bias[n];
+                else if constexpr (EPI == 2) *o = v + bias[n];
+                else *o += alpha * bias[n] * v;
             }
         }
     }
@@ -314,7 +321,7 @@ template <typename D>
 __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const typename D::storage *kpool, const typename D::storage *vpool,
                                                        const int32_t *row_seq, const int32_t *row_pos, const int32_t *seq_slot,
                                                        const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
-                                                       float scale, int sink, const float *gate, int ldg, typename D::storage *out, int ldo) {
+                                                       float scale, int sink, const float *gate, int ldg, typename D::storage *out, int ldo, int v_row) {
     extern __shared__ float smem[];
     float *qs = smem;        // [dim]
     float *ps = smem + dim;  // [64]
@@ -347,7 +354,7 @@ __global__ __launch_bounds__(64) void attn_rows_kernel(const float *qbuf, const 
         for (int i = 0; i < 8; ++i) acc[i] *= corr;
         for (int jj = 0; jj < cnt; ++jj) {
             const int jg = kb + jj;
-            const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * G + g) * page_size + jg % page_size) * vdim;
+            const typename D::storage *vr = vpool + (((size_t)bt[jg / page_size] * G + g) * page_size + jg % page_size) * v_row;
             const float pj = ps[jj];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -384,7 +391,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                                                         const int32_t *block_table, int max_pages, int page_size, int H, int G, int dim, int vdim,
                                                         float scale, int sink, int HGB, int n_hblk, int keys_per_split, int n_splits, const float *gate,
                                                         int ldg, typename D::storage *out, int ldo, float *part_acc, float *part_ml, int page_shift,
-                                                        int vec_ok) {
+                                                        int vec_ok, int v_row) {
     using S = typename D::storage;
     extern __shared__ float smem[];
     // LDS rows as wide as the template: zeros behind dim / vdim, no guards in the product loops.  bfloat16 pages: the K tile stays bfloat16
@@ -459,8 +466,8 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(const float *qbuf, const
                 for (int e = 0; e < 8; ++e) raw[it][e] = (S)0;
                 if (pl >= 0 && j < k_end && c8 < (is_v ? vdim : dim)) {
                     const int pg = page_shift >= 0 ? (j >> page_shift) : (j / page_size), in_pg = j - pg * page_size;
-                    const int wd = is_v ? vdim : dim;
-                    const S *src = (is_v ? vpool : kpool) + (((size_t)bt[pg] * G + kvh) * page_size + in_pg) * wd + c8;
+                    const int wd = is_v ? vdim : dim;  // v_row: the width of a row of vpool (vdim, or the key row's when the values are its leading columns)
+                    const S *src = (is_v ? vpool : kpool) + (((size_t)bt[pg] * G + kvh) * page_size + in_pg) * (is_v ? v_row : dim) + c8;
                     if (vec_ok) {  // (widths are multiples of 8: a chunk is whole or absent)
                         if constexpr (sizeof(S) == 2) *reinterpret_cast<u32x4 *>(raw[it]) = *reinterpret_cast<const u32x4 *>(src);
                         else {
@@ -863,6 +870,348 @@ __global__ __launch_bounds__(64) void delta_out_kernel(const float *obuf, const 
     const float inv = 1.f / sqrtf(ss / (float)vdim + eps);
     for (int c = lane; c < vdim; c += 64)
         out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o[c] * inv * w[c] * silu_f(gate[(size_t)t * ldg + (size_t)h * vdim + c]));
+}
+
+// ---- Dynamic Tanh norm of float32 rows -> D rows: tanh(alpha x) * w + b (no statistics of the row).  rows_idx: optional gather. ----
+template <typename D>
+__global__ void dyt_kernel(const float *x, const float *w, const float *b, float alpha, typename D::storage *out, int width, const int32_t *rows_idx) {
+    const int r = blockIdx.x;
+    const float *src = x + (size_t)(rows_idx ? rows_idx[r] : r) * width;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)r * width + c] = D::from_float(tanhf(alpha * src[c]) * w[c] + b[c]);
+}
+
+// ---- RMS norm of n columns of float32 rows (a latent) -> D rows: x / sqrt(mean x^2 + eps) * w.  One wave per row. ----------------
+template <typename D>
+__global__ __launch_bounds__(64) void rms_cols_kernel(const float *in, int ldi, int n, const float *w, float eps, typename D::storage *out, int ldo) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float *src = in + (size_t)t * ldi;
+    float ss = 0.f;
+    for (int c = lane; c < n; c += 64) ss += src[c] * src[c];
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)n + eps);
+    for (int c = lane; c < n; c += 64) out[(size_t)t * ldo + c] = D::from_float(src[c] * inv * w[c]);
+}
+
+// ---- latent attention, step 1.  Queries q [rows, H, dim + rot] (float32): the plain part -> qn (D, the input of the per-head key
+// absorption), the rotated part -> qbuf[t, h, rank ..] after its rotation.  With own_kv (the layer has its own latent projection, columns
+// kv0 .. of proj: rank latent columns, then rot columns of one rotated key part shared by all heads): the latent is RMS-normed with
+// its weight and appended to the sequence's page row [c (rank) | rotated key part (rot)] -- the whole K/V cache of the layer.
+// Rotation: pair (2i, 2i+1) by pos * freq[i], cos and sin times mult.  grid (rows, H + 1), one wave each.
+template <typename D>
+__global__ __launch_bounds__(64) void latent_prep_kernel(const float *q, int H, int dim, int rot, int rank, const float *proj, int ldp, int kv0,
+                                                         const float *c_norm, float eps, int own_kv, const int32_t *row_seq, const int32_t *row_pos,
+                                                         const int32_t *seq_slot, const int32_t *block_table, int max_pages, int page_size,
+                                                         const float *freq, int rot_dims, float mult, typename D::storage *qn, float *qbuf,
+                                                         typename D::storage *pool) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int pos = row_pos[t];
+    auto turn = [&](const float *src, int p, float &u, float &v) {
+        const int c = 2 * p;
+        u = src[c], v = (c + 1 < rot) ? src[c + 1] : 0.f;
+        if (c + 1 < rot_dims) {
+            float sn, cs;
+            sincosf((float)pos * freq[p], &sn, &cs);
+            sn *= mult, cs *= mult;
+            const float nu = u * cs - v * sn, nv = v * cs + u * sn;
+            u = nu, v = nv;
+        }
+    };
+    if (hh < H) {
+        const float *src = q + ((size_t)t * H + hh) * (dim + rot);
+        for (int c = lane; c < dim; c += 64) qn[((size_t)t * H + hh) * dim + c] = D::from_float(src[c]);
+        float *dst = qbuf + ((size_t)t * H + hh) * (rank + rot) + rank;
+        for (int p = lane; 2 * p < rot; p += 64) {
+            float u, v;
+            turn(src + dim, p, u, v);
+            dst[2 * p] = u;
+            if (2 * p + 1 < rot) dst[2 * p + 1] = v;
+        }
+        return;
+    }
+    if (!own_kv) return;
+    const int slot = seq_slot[row_seq[t]];
+    const int page = block_table[(size_t)slot * max_pages + pos / page_size], in_page = pos % page_size;
+    typename D::storage *dst = pool + ((size_t)page * page_size + in_page) * (rank + rot);
+    const float *src = proj + (size_t)t * ldp + kv0;
+    float ss = 0.f;
+    for (int c = lane; c < rank; c += 64) ss += src[c] * src[c];
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)rank + eps);
+    for (int c = lane; c < rank; c += 64) dst[c] = D::from_float(src[c] * inv * c_norm[c]);
+    for (int p = lane; 2 * p < rot; p += 64) {
+        float u, v;
+        turn(src + rank, p, u, v);
+        dst[rank + 2 * p] = D::from_float(u);
+        if (2 * p + 1 < rot) dst[rank + 2 * p + 1] = D::from_float(v);
+    }
+}
+
+// ---- out[t, c] = in[t, c] * gate(g[t, c]) as D rows.  kind 0: sigmoid, 1: SiLU ----------------------------------------------------
+template <typename D>
+__global__ void gate_mul_kernel(const float *in, int ldi, const float *g, int ldg, int n, int kind, typename D::storage *out, int ldo, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * n) return;
+    const int t = (int)(i / n), c = (int)(i % n);
+    const float z = g[(size_t)t * ldg + c];
+    out[(size_t)t * ldo + c] = D::from_float(in[(size_t)t * ldi + c] * (kind == 0 ? sigmoid_f(z) : silu_f(z)));
+}
+
+// ---- gated feed-forward activation: cat[t, col0 + c] = act(proj[t, g0 + c]) * proj[t, u0 + c] ------------------------------------
+template <typename D>
+__global__ void ff_gated_act_kernel(const float *proj, int ldp, int g0, int u0, int ff, int kind, typename D::storage *out, int ldo, int col0, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * ff) return;
+    const int t = (int)(i / ff), c = (int)(i % ff);
+    out[(size_t)t * ldo + col0 + c] = D::from_float(act_f(proj[(size_t)t * ldp + g0 + c], kind) * proj[(size_t)t * ldp + u0 + c]);
+}
+
+// ---- linear recurrences with a decaying matrix state --------------------------------------------------------------------------------
+// log-sigmoid without overflow
+__device__ __forceinline__ float logsigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+// Exponential gates with a running maximum (mLSTM).  Per (sequence, head), token by token:
+//   li = cap tanh((x_i + b_i) / cap),  lf = logsigmoid(cap tanh((x_f + b_f) / cap)),  m' = max(lf + m, li)
+//   decay a = exp(lf + m - m'),  input scale b = exp(li - m'),  floor e = exp(-m')       (m starts at 0 with the sequence)
+// m -> max(m + A, B) composes associatively ((A1, B1) then (A2, B2) = (A1 + A2, max(B1 + A2, B2))), so a wave scans 64 tokens at a time.
+// proj columns i0 + h / f0 + h hold x_i / x_f.  gates: [rows, H, 3] = (a, b, e).  m_state: [slots, H].
+__global__ __launch_bounds__(64) void expgate_scan_kernel(const float *proj, int ldp, int i0, int f0, const float *i_bias, const float *f_bias, float cap,
+                                                          const int32_t *seq_row0, const int32_t *seq_slot, float *m_state, float *gates, int H) {
+    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
+    float m = m_state[(size_t)slot * H + h];
+    for (int t0 = 0; t0 < n; t0 += 64) {
+        const int t = t0 + lane;
+        const bool ok = t < n;
+        float li = 0.f, lf = 0.f;
+        if (ok) {
+            const float *row = proj + (size_t)(r0 + t) * ldp;
+            li = cap * tanhf((row[i0 + h] + i_bias[h]) / cap);
+            lf = logsigmoid_f(cap * tanhf((row[f0 + h] + f_bias[h]) / cap));
+        }
+        float A = ok ? lf : 0.f, B = ok ? li : -INFINITY;  // lanes past the end: the identity
+        for (int off = 1; off < 64; off <<= 1) {
+            const float pa = __shfl_up(A, off, 64), pb = __shfl_up(B, off, 64);
+            if (lane >= off) {
+                B = fmaxf(pb + A, B);
+                A = pa + A;
+            }
+        }
+        const float m_t = fmaxf(m + A, B);
+        float m_prev = __shfl_up(m_t, 1, 64);
+        if (lane == 0) m_prev = m;
+        if (ok) {
+            float *g = gates + ((size_t)(r0 + t) * H + h) * 3;
+            g[0] = expf(lf + m_prev - m_t);
+            g[1] = expf(li - m_t);
+            g[2] = expf(-m_t);
+        }
+        m = __shfl(m_t, min(63, n - 1 - t0), 64);
+    }
+    if (lane == 0) m_state[(size_t)slot * H + h] = m;
+}
+
+// decay per key channel (gated linear attention): z[t, c] <- sigmoid(z + bias[c])^(1/tau) = exp(logsigmoid(z + bias) / tau), in place
+__global__ void channel_decay_kernel(float *z, const float *bias, int n, float inv_tau, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * n) return;
+    z[i] = expf(logsigmoid_f(z[i] + bias[i % n]) * inv_tau);
+}
+// float32 columns of proj -> D rows (the input of a second, low-rank projection)
+template <typename D>
+__global__ void cast_cols_kernel(const float *in, int ldi, int c0, int n, typename D::storage *out, int ldo, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * n) return;
+    const int t = (int)(i / n), c = (int)(i % n);
+    out[(size_t)t * ldo + c] = D::from_float(in[(size_t)t * ldi + c0 + c]);
+}
+
+// The recurrence itself, token by token:   S <- diag(a_t) S + b_t k_t v_t^T;   o_t = S^T q_t      (S: [key_dim, columns] per head, float32)
+//   CHAN false: a_t one number per head (gates[.., 0]), b_t = gates[.., 1]     CHAN true: a_t per key channel (decay[t, h, d]), b_t = 1
+// ones != 0 appends one column whose value is 1 for every token: it carries the normaliser n_t = a n + b k, read out as n_t . q_t.
+// grid (heads, sequences, blocks of 256 / LPC columns), 256 threads; LPC lanes share a column, RPT key rows each in registers (as delta_kernel).
+// q | k | v at columns q0 | k0 | v0 of proj (head-major).  State [slot, head, column, key_dim].  obuf [rows, H, VE], VE = vdim + ones.
+template <int RPT, int LPC, bool CHAN>
+__global__ __launch_bounds__(256) void linrec_kernel(const float *proj, int ldp, int q0, int k0, int v0, const float *gates, const float *decay,
+                                                     const int32_t *seq_row0, const int32_t *seq_slot, float *state, float *obuf, int H, int dim,
+                                                     int vdim, int ones) {
+    constexpr int DP = LPC * RPT, CPB = 256 / LPC;
+    constexpr int TB = 4096 / DP < 32 ? 4096 / DP : 32;
+    __shared__ float qs[TB * DP], ks[TB * DP], as[CHAN ? TB * DP : TB], vs[TB * CPB], bs[TB], os[TB * CPB];
+    const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * CPB, VE = vdim + ones;
+    const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
+    const int tid = threadIdx.x, jl = tid / LPC, r = tid % LPC, j = j0 + jl;
+    const bool active = j < VE;
+    float S[RPT];
+    float *sp = state + (((size_t)slot * H + h) * VE + (active ? j : 0)) * dim + r * RPT;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) S[i] = (active && r * RPT + i < dim) ? sp[i] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += TB) {
+        const int nt = min(TB, n - t0);
+        __syncthreads();
+        for (int i = tid; i < TB * DP; i += 256) {
+            const int tt = i / DP, d = i % DP;
+            const bool ok = tt < nt && d < dim;
+            const float *row = proj + (size_t)(r0 + t0 + (ok ? tt : 0)) * ldp + (size_t)h * dim + d;
+            qs[i] = ok ? row[q0] : 0.f;
+            ks[i] = ok ? row[k0] : 0.f;
+            if constexpr (CHAN) as[i] = ok ? decay[((size_t)(r0 + t0 + tt) * H + h) * dim + d] : 1.f;
+        }
+        for (int i = tid; i < TB * CPB; i += 256) {
+            const int tt = i / CPB, c = j0 + i % CPB;
+            vs[i] = (tt < nt && c < VE) ? (c < vdim ? proj[(size_t)(r0 + t0 + tt) * ldp + v0 + (size_t)h * vdim + c] : 1.f) : 0.f;
+        }
+        if (tid < TB) {
+            const bool ok = tid < nt;
+            if constexpr (!CHAN) as[tid] = ok ? gates[((size_t)(r0 + t0 + tid) * H + h) * 3] : 1.f;
+            bs[tid] = ok ? (CHAN ? 1.f : gates[((size_t)(r0 + t0 + tid) * H + h) * 3 + 1]) : 0.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float bv = bs[tt] * vs[tt * CPB + jl];
+            const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT;
+            float a_s = 1.f;
+            if constexpr (!CHAN) a_s = as[tt];
+            float od0 = 0.f, od1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) {
+                float a = a_s;
+                if constexpr (CHAN) a = as[tt * DP + r * RPT + i];
+                S[i] = S[i] * a + kt[i] * bv;
+                if (i & 1) od1 += S[i] * qt[i];
+                else od0 += S[i] * qt[i];
+            }
+            const float od = column_sum<LPC>(od0 + od1, tid);
+            if (r == 0) os[tt * CPB + jl] = od;
+        }
+        __syncthreads();
+        for (int i = tid; i < nt * CPB; i += 256) {
+            const int tt = i / CPB, c = i % CPB;
+            if (j0 + c < VE) obuf[((size_t)(r0 + t0 + tt) * H + h) * VE + j0 + c] = os[i];
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int i = 0; i < RPT; ++i)
+            if (r * RPT + i < dim) sp[i] = S[i];
+    }
+}
+
+// read-out of a linear recurrence, one wave per (row, head):  o = obuf[t, h, :vdim] * qscale;  with ones: o /= max(|n.q|, e) + 1e-6 where n.q is
+// the appended column (times qscale) and e the gate floor;  then o / rms(o) * w[h * w_stride + c] * gate(g)   (gate_kind 0 sigmoid, 1 SiLU)
+template <typename D>
+__global__ __launch_bounds__(64) void linrec_out_kernel(const float *obuf, int VE, int ones, const float *gates, float qscale, const float *w,
+                                                        int w_stride, float eps, const float *gate, int ldg, int gate_kind, int H, int vdim,
+                                                        typename D::storage *out, int ldo) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float *o = obuf + ((size_t)t * H + h) * VE;
+    float mul = qscale;
+    if (ones) mul = qscale / (fmaxf(fabsf(o[vdim] * qscale), gates[((size_t)t * H + h) * 3 + 2]) + 1e-6f);
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += 64) {
+        const float v = o[c] * mul;
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float inv = mul / sqrtf(ss / (float)vdim + eps);
+    for (int c = lane; c < vdim; c += 64) {
+        const float z = gate[(size_t)t * ldg + (size_t)h * vdim + c];
+        out[(size_t)t * ldo + (size_t)h * vdim + c] = D::from_float(o[c] * inv * w[(size_t)h * w_stride + c] * (gate_kind == 0 ? sigmoid_f(z) : silu_f(z)));
+    }
+}
+
+// ---- mixture of experts: routing and activation, one workgroup per row -----------------------------------------------------------------
+// proj columns of the row: router logits z [ET] at r0 (ET = experts + identity experts) | shared gate (1) at sg0 | shared up [ffs] at su0 |
+// expert e's up [ffe] at eu0 + e * ffe.  s = softmax(z); choice = s + correction; the experts form `groups` equal runs of neighbours, a
+// group scores its largest choice, only the `keep` best groups can be taken; the `top` largest choices among them are taken (ties: the lower
+// index); weights are their s, not renormalised.  The last `identity` experts return their input: their weights are summed into idw[t].
+// cat row: [ sigmoid(sg) * relu(up)^2  (ffs) | w_e * relu(up_e)^2 (ffe each; 0 for experts not taken) ].
+template <typename D>
+__global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, int ldp, int r0, int sg0, int su0, int eu0, int experts, int identity, int top,
+                                                            int groups, int keep, int ffe, int ffs, const float *correction,
+                                                            typename D::storage *out, int ldo, int col0, float *idw) {
+    __shared__ float sw[256], sc[256];
+    __shared__ float gm[256];
+    const int t = blockIdx.x, tid = threadIdx.x, ET = experts + identity;
+    const float *row = proj + (size_t)t * ldp;
+    if (tid < 64) {  // one wave routes (ET <= 256: four experts a lane at most)
+        float z[4], mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 64 * i;
+            z[i] = e < ET ? row[r0 + e] : -INFINITY;
+            mx = fmaxf(mx, z[i]);
+        }
+        mx = wave_max(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            z[i] = (tid + 64 * i) < ET ? expf(z[i] - mx) : 0.f;
+            sum += z[i];
+        }
+        sum = wave_sum(sum);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = tid + 64 * i;
+            if (e < ET) {
+                const float s = z[i] / sum;
+                sw[e] = s;
+                sc[e] = s + correction[e];
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {  // groups, then the top choices: a few dozen comparisons
+        const int per = ET / groups;
+        for (int g = 0; g < groups; ++g) {
+            float m = -INFINITY;
+            for (int e = g * per; e < (g + 1) * per; ++e) m = fmaxf(m, sc[e]);
+            gm[g] = m;
+        }
+        for (int g = 0; g < groups; ++g) {  // rank of the group: how many beat it (ties: the lower index first)
+            int rank = 0;
+            for (int o = 0; o < groups; ++o) rank += (gm[o] > gm[g]) || (gm[o] == gm[g] && o < g);
+            if (rank >= keep)
+                for (int e = g * per; e < (g + 1) * per; ++e) sc[e] = -INFINITY;
+        }
+    }
+    __syncthreads();
+    float wgt = 0.f;
+    bool dead = true;
+    if (tid < ET) {
+        const float c = sc[tid];
+        dead = c == -INFINITY && true;
+        int rank = 0;
+        for (int o = 0; o < ET; ++o) rank += (sc[o] > c) || (sc[o] == c && o < tid);
+        wgt = (rank < top && !(c == -INFINITY)) ? sw[tid] : 0.f;
+    }
+    (void)dead;
+    __syncthreads();
+    if (tid < ET) sw[tid] = wgt;
+    __syncthreads();
+    if (tid == 0) {
+        float a = 0.f;
+        for (int e = experts; e < ET; ++e) a += sw[e];
+        idw[t] = a;
+    }
+    const float sgate = ffs > 0 ? sigmoid_f(row[sg0]) : 0.f;
+    typename D::storage *o = out + (size_t)t * ldo + col0;
+    for (int c = tid; c < ffs; c += 256) {
+        const float u = fmaxf(row[su0 + c], 0.f);
+        o[c] = D::from_float(sgate * u * u);
+    }
+    const int n = experts * ffe;
+    for (int c = tid; c < n; c += 256) {
+        const float w = sw[c / ffe], u = fmaxf(row[eu0 + c], 0.f);
+        o[ffs + c] = D::from_float(w * u * u);
+    }
+}
+// identity experts: x[t, c] += ls[c] * idw[t] * h[t, c]  (ls may be null: 1)
+template <typename D>
+__global__ void identity_axpy_kernel(float *x, const typename D::storage *h, const float *idw, const float *ls, float mult, int width, int rows) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * width) return;
+    const int t = (int)(i / width), c = (int)(i % width);
+    x[i] += mult * (ls ? ls[c] : 1.f) * idw[t] * D::to_float(h[i]);
 }
 
 // ---- small helpers -----------------------------------------------------------------------------------------------------------

@@ -22,9 +22,12 @@ _lib = ctypes.CDLL(str(_LIB_PATH), mode=os.RTLD_LOCAL if hasattr(os, "RTLD_LOCAL
 _vp, _i, _f, _sz, _l = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t, ctypes.c_long
 _P = ctypes.POINTER
 
-MIX_ATTENTION, MIX_DELTA = 0, 1
+MIX_ATTENTION, MIX_DELTA, MIX_LINREC, MIX_LATENT = 0, 1, 2, 3
+REC_CHANNEL, REC_EXPGATE = 0, 1
+NORM_RMS, NORM_DYT = 0, 1
+FF_PLAIN, FF_GATED, FF_MOE = 0, 1, 2
 HY_F32, HY_BF16 = 0, 2
-FF_GELU_ERF, FF_GELU_TANH, FF_SILU = 0, 1, 2
+FF_GELU_ERF, FF_GELU_TANH, FF_SILU, FF_RELU2 = 0, 1, 2, 3
 
 
 class TlHybridLayer(ctypes.Structure):
@@ -32,7 +35,16 @@ class TlHybridLayer(ctypes.Structure):
                 ("w_in_dev", _vp), ("w_out_dev", _vp), ("norm_dev", _vp), ("norm_offset", _f),
                 ("rot_dims", _i), ("rot_base", _f), ("scale", _f), ("qk_unit_rms", _i), ("sink", _i), ("gated", _i),
                 ("conv_taps", _i), ("conv_dev", _vp), ("a_log_dev", _vp), ("dt_bias_dev", _vp), ("out_norm_dev", _vp),
-                ("unit_eps", _f)]
+                ("unit_eps", _f),
+                ("norm_kind", _i), ("norm_alpha", _f), ("norm2_alpha", _f), ("norm_bias_dev", _vp), ("norm2_bias_dev", _vp),
+                ("norm2_dev", _vp), ("w_in2_dev", _vp), ("w_out2_dev", _vp), ("ls1_dev", _vp), ("ls2_dev", _vp), ("ff_kind", _i),
+                ("experts", _i), ("identity", _i), ("top", _i), ("groups", _i), ("keep", _i), ("expert_ff", _i), ("shared_ff", _i),
+                ("correction_dev", _vp),
+                ("rec_kind", _i), ("gate_cap", _f), ("tau", _f), ("a_rank", _i), ("a2_dev", _vp), ("a2_bias_dev", _vp),
+                ("i_bias_dev", _vp), ("f_bias_dev", _vp),
+                ("q_rank", _i), ("kv_rank", _i), ("rot_dim", _i), ("kv_from", _i), ("dq_norm_dev", _vp), ("dkv_norm_dev", _vp),
+                ("uq_dev", _vp), ("uk_t_dev", _vp), ("uv_dev", _vp),
+                ("rot_factor", _f), ("rot_original", _f), ("rot_fast", _f), ("rot_slow", _f)]
 
 
 class TlHybridConfig(ctypes.Structure):
@@ -40,6 +52,7 @@ class TlHybridConfig(ctypes.Structure):
                 ("parallel_block", _i), ("loop_start", _i), ("loop_stop", _i), ("loop_times", _i),
                 ("loop_in_dev", _vp), ("loop_step_dev", _vp), ("embed_dev", _vp), ("final_norm_dev", _vp),
                 ("final_norm_offset", _f), ("head_dev", _vp),
+                ("embed_scale", _f), ("final_norm_kind", _i), ("final_norm_alpha", _f), ("final_norm_bias_dev", _vp),
                 ("page_size", _i), ("num_pages", _i), ("max_slots", _i), ("max_pages_per_seq", _i), ("max_rows", _i)]
 
 

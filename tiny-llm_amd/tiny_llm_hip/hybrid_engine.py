@@ -18,7 +18,11 @@ from .layer_list import LayerListConfig, pack_layer_list
 
 __all__ = ["HybridEngine"]
 
-_FF_ACT = {"gelu_erf": 0, "gelu_tanh": 1, "silu": 2}
+_FF_ACT = {"gelu_erf": 0, "gelu_tanh": 1, "silu": 2, "relu2": 3}
+_MIX = {"attention": 0, "delta": 1, "linrec": 2, "latent": 3}
+_REC = {"channel": 0, "expgate": 1}
+_NORM = {"rms": 0, "dyt": 1}
+_FF_KIND = {"plain": 0, "gated": 1, "moe": 2}
 
 
 class HybridEngine:
@@ -45,12 +49,15 @@ class HybridEngine:
         self.page_size, self.max_batch, self.vocab_size = int(page_size), int(max_batch), cfg.vocab
         self.max_prefill_rows = max(int(max_prefill_rows), self.max_batch)
         self.num_hidden_layers = len(cfg.layers)
-        self.has_recurrent_state = any(L.kind == "delta" for L in cfg.layers)
+        self.has_recurrent_state = any(L.kind in ("delta", "linrec") for L in cfg.layers)
+        for i, L in enumerate(cfg.layers):  # a size the configuration leaves to the tensors
+            if L.a_rank < 0:
+                L.a_rank = int(model.tensors[cfg.prefix(i) + "mix.a1"].shape[0])
         w = self._weights = pack_layer_list(cfg, model.tensors, dtype, self.device)
         layers = (ext.TlHybridLayer * len(cfg.layers))()
         for i, (L, t) in enumerate(zip(cfg.layers, w["layers"])):
             s = layers[i]
-            s.kind = ext.MIX_ATTENTION if L.kind == "attention" else ext.MIX_DELTA
+            s.kind = _MIX[L.kind]
             s.heads, s.kv_heads, s.dim, s.vdim, s.ff, s.ff_act = L.heads, L.kv_heads, L.dim, L.vdim, L.ff, _FF_ACT[L.ff_act]
             s.w_in_dev, s.w_out_dev, s.norm_dev, s.norm_offset = t["w_in"].data_ptr(), t["w_out"].data_ptr(), t["norm"].data_ptr(), cfg.norm_offset
             s.rot_dims, s.rot_base, s.scale = L.rot_dims, L.rot_base, L.scale
@@ -59,9 +66,27 @@ class HybridEngine:
             if L.kind == "delta":
                 s.conv_dev, s.a_log_dev, s.dt_bias_dev, s.out_norm_dev = (t["conv"].data_ptr(), t["a_log"].data_ptr(),
                                                                           t["dt_bias"].data_ptr(), t["out_norm"].data_ptr())
+            ptr = lambda key: t[key].data_ptr() if key in t else None
+            s.norm_kind, s.norm_alpha, s.norm2_alpha = _NORM[cfg.norm_kind], t.get("norm_alpha", 0.0), t.get("norm2_alpha", 0.0)
+            s.norm_bias_dev, s.norm2_bias_dev, s.norm2_dev = ptr("norm_bias"), ptr("norm2_bias"), ptr("norm2")
+            s.w_in2_dev, s.w_out2_dev, s.ls1_dev, s.ls2_dev = ptr("w_in2"), ptr("w_out2"), ptr("ls1"), ptr("ls2")
+            s.ff_kind, s.experts, s.identity, s.top, s.groups, s.keep = _FF_KIND[L.ff_kind], L.experts, L.identity, L.top, L.groups, L.keep
+            s.expert_ff, s.shared_ff, s.correction_dev = L.expert_ff, L.shared_ff, ptr("correction")
+            s.kv_from = -1
+            if L.kind == "linrec":
+                s.rec_kind, s.gate_cap, s.tau, s.a_rank, s.out_norm_dev = _REC[L.rec_kind], L.gate_cap, L.tau, max(L.a_rank, 0), t["out_norm"].data_ptr()
+                s.a2_dev, s.a2_bias_dev, s.i_bias_dev, s.f_bias_dev = ptr("a2"), ptr("a2_bias"), ptr("i_bias"), ptr("f_bias")
+            elif L.kind == "latent":
+                s.q_rank, s.kv_rank, s.rot_dim, s.kv_from = L.q_rank, L.kv_rank, L.rot_dim, L.kv_from
+                s.dq_norm_dev, s.dkv_norm_dev, s.uq_dev, s.uk_t_dev, s.uv_dev = ptr("dq_norm"), ptr("dkv_norm"), ptr("uq"), ptr("uk_t"), ptr("uv")
+                if L.rot_scaling:
+                    s.rot_factor, s.rot_original, s.rot_fast, s.rot_slow = L.rot_scaling
         c = ext.TlHybridConfig()
         c.dtype = ext.HY_BF16 if dtype == torch.bfloat16 else ext.HY_F32
-        c.width, c.vocab, c.num_layers, c.norm_eps, c.residual_mult, c.parallel_block = cfg.width, cfg.vocab, len(cfg.layers), cfg.norm_eps, cfg.residual_mult, 1
+        c.width, c.vocab, c.num_layers, c.norm_eps, c.residual_mult = cfg.width, cfg.vocab, len(cfg.layers), cfg.norm_eps, cfg.residual_mult
+        c.parallel_block, c.embed_scale = int(cfg.block == "parallel"), cfg.embed_scale
+        c.final_norm_kind, c.final_norm_alpha = _NORM[cfg.norm_kind], w.get("final_norm_alpha", 0.0)
+        c.final_norm_bias_dev = w["final_norm_bias"].data_ptr() if "final_norm_bias" in w else None
         if cfg.loop:
             c.loop_start, c.loop_stop, c.loop_times = cfg.loop
             c.loop_in_dev, c.loop_step_dev = w["loop_in"].data_ptr(), w["loop_step"].data_ptr()

@@ -5,7 +5,7 @@ A *family* turns a checkpoint's ``config.json`` into a ``LayerListConfig`` and n
 registry ``loader.load_weights`` and ``models.engine_for`` consult (key: config.json's ``architecture``).  The engine itself
 knows mixer kinds and their options, not families.
 
-Fonapel (the one family so far) -- per layer, with h = norm(x) and one norm for both branches:
+Fonapel -- per layer, with h = norm(x) and one norm for both branches:
 
     x <- x + m * (mixer(h) + ff(h))            norm: x / sqrt(mean x^2 + eps) * (1 + w)
     ff(h) = W_down gelu_erf(W_up h)
@@ -21,6 +21,26 @@ Fonapel (the one family so far) -- per layer, with h = norm(x) and one norm for 
 
     loop {start, stop, times}: layers start..stop-1 run `times` times with the same weights and separate caches; each pass
         is entered through x <- W_in [x ; x0] + step[t] (x0 = the embedding output).
+
+Zefapel -- x = embed[token] * embedding.scale; per layer, sequentially, with Dynamic Tanh norms dyt(x) = tanh(alpha x) w + b and
+per-channel layer scales ls1 / ls2:
+
+    x <- x + ls1 * W_o mixer(dyt1(x));   x <- x + ls2 * ff(dyt2(x))
+
+    mixer "mlstm": q (* dim^-1/2), k, v per head; log gates i = cap tanh((W_i h + b_i) / cap), f = logsigmoid(cap tanh((W_f h + b_f) / cap));
+        m' = max(f + m, i) (m starts at 0);  S <- e^(f+m-m') S + e^(i-m') k v^T;  n likewise with k;
+        o = S^T q / (max(|n.q|, e^-m') + 1e-6);  o / rms(o) * norm * sigmoid(W_g h).
+    mixer "gla": the same state with a decay per key channel, a = sigmoid(W_a2 W_a1 h + b)^(1/tau), no gates, no normaliser;
+        rms_norm(o) * norm[vdim] * silu(W_g h).
+    mixer "latent_attention": q = W_uq rms_norm(W_dq h); W_dkv h = [latent (kv_rank) | one rotated key part (rot_dim)], the latent
+        RMS-normed; per head k = [W_uk c | rotated part], v = W_uv c, q = [plain (dim) | rotated (rot_dim)]; rotation of adjacent pairs with
+        frequencies rescaled by rot.scaling (factor, original, fast, slow) and cos / sin times 0.1 ln(factor) + 1; causal softmax
+        of q.k * scale; heads * sigmoid(W_g h).  Only [c | rotated part] is cached; "kv_from": j reads layer j's cache instead of
+        projecting its own.
+    ff "dense": W_down (silu(W_gate h) * W_up h).
+    ff "moe": s = softmax(W_router h) over experts + identity experts; choice = s + correction; experts form groups.count runs of
+        neighbours, the groups.keep groups with the largest choice stay; the `top` largest choices among them are taken with weight s
+        (not renormalised); expert = W_down relu(W_up h)^2, identity expert = h; plus sigmoid(W_sg h) * shared expert.
 """
 
 from __future__ import annotations
@@ -30,12 +50,12 @@ from typing import Any, Callable
 
 import torch
 
-__all__ = ["LayerSpec", "LayerListConfig", "FAMILIES", "fonapel_config", "pack_layer_list"]
+__all__ = ["LayerSpec", "LayerListConfig", "FAMILIES", "fonapel_config", "zefapel_config", "pack_layer_list"]
 
 
 @dataclass
 class LayerSpec:
-    kind: str                       # "attention" | "delta"
+    kind: str                       # "attention" | "delta" | "linrec" | "latent"
     heads: int
     kv_heads: int
     dim: int
@@ -52,6 +72,26 @@ class LayerSpec:
     # delta
     conv_taps: int = 0
     unit_eps: float = 1e-6
+    # feed-forward: "plain" W_down act(W_up h) | "gated" W_down (act(W_gate h) * W_up h) | "moe"
+    ff_kind: str = "plain"
+    experts: int = 0
+    identity: int = 0               # identity experts behind the real ones in the router's output
+    top: int = 0
+    groups: int = 1
+    keep: int = 1
+    expert_ff: int = 0
+    shared_ff: int = 0
+    # linrec: "channel" (a decay per key channel, rank-`a_rank` projection pair, temperature tau) | "expgate" (capped exponential gates)
+    rec_kind: str = "channel"
+    gate_cap: float = 0.0
+    tau: float = 1.0
+    a_rank: int = 0
+    # latent attention
+    q_rank: int = 0
+    kv_rank: int = 0
+    rot_dim: int = 0
+    kv_from: int = -1               # layer whose latent cache is read; -1: the layer's own
+    rot_scaling: tuple[float, float, float, float] | None = None  # (factor, original, fast, slow)
 
 
 @dataclass
@@ -64,6 +104,10 @@ class LayerListConfig:
     layers: list[LayerSpec]
     norm_offset: float = 1.0        # norm weights stored around zero are applied as (1 + w)
     loop: tuple[int, int, int] | None = None  # (start, stop, times)
+    norm_kind: str = "rms"          # "rms" | "dyt" (tanh(alpha x) w + b: tensors <name>, <name>.alpha, <name>.b)
+    block: str = "parallel"         # "parallel": x += m (mixer(h) + ff(h)), one norm | "sequential": two norms, two residual sums
+    layer_scale: bool = False       # sequential block: per-channel vectors ls1 / ls2 on the branches
+    embed_scale: float = 1.0
     prefix: Callable[[int], str] = field(default=lambda i: f"l{i}.")
 
     @property
@@ -132,40 +176,174 @@ def _fonapel_tensor_shapes(cfg: LayerListConfig) -> dict[str, tuple[int, ...]]:
     return want
 
 
+def zefapel_config(config: dict) -> LayerListConfig:
+    """config.json of a Zefapel checkpoint -> LayerListConfig.  Every size and every constant the file gives is read from it."""
+    for key in ("layers", "norm", "embedding", "vocab", "width"):
+        if key not in config:
+            raise ValueError(f"config.json lacks {key!r}")
+    layers = []
+    for i, entry in enumerate(config["layers"]):
+        kind, mc, mlp = entry.get("type"), entry.get("mixer") or {}, entry.get("mlp")
+        ff: dict[str, Any] = {}
+        if mlp is not None:
+            if mlp.get("kind") == "dense":
+                ff = dict(ff=int(mlp["ff"]), ff_kind="gated", ff_act="silu")
+            elif mlp.get("kind") == "moe":
+                r, shared = mlp["router"], mlp.get("shared")
+                experts, expert_ff = int(r["experts"]), int(mlp["expert"]["ff"])
+                shared_ff = int(shared["ff"]) if shared else 0
+                groups = r.get("groups") or {"count": 1, "keep": 1}
+                ff = dict(ff=shared_ff + experts * expert_ff, ff_kind="moe", ff_act="relu2", experts=experts, identity=int(r.get("identity", 0)),
+                          top=int(r["top"]), groups=int(groups["count"]), keep=int(groups["keep"]), expert_ff=expert_ff, shared_ff=shared_ff)
+                if (experts + ff["identity"]) % ff["groups"]:
+                    raise ValueError(f"layer {i}: {experts} + {ff['identity']} router outputs do not form {ff['groups']} equal groups")
+            else:
+                raise ValueError(f"layer {i}: unsupported mlp.kind={mlp.get('kind')!r}")
+        heads, dim, vdim = int(mc["heads"]), int(mc["dim"]), int(mc["vdim"])
+        if kind == "mlstm":
+            layers.append(LayerSpec(kind="linrec", rec_kind="expgate", heads=heads, kv_heads=heads, dim=dim, vdim=vdim, gate_cap=float(mc["gate_cap"]), **ff))
+        elif kind == "gla":
+            layers.append(LayerSpec(kind="linrec", rec_kind="channel", heads=heads, kv_heads=heads, dim=dim, vdim=vdim, tau=float(mc["tau"]),
+                                    a_rank=-1, **ff))  # the rank is the first projection's row count: taken from the tensor
+        elif kind == "latent_attention":
+            rot, sc = mc.get("rot") or {}, None
+            if rot.get("scaling"):
+                g = rot["scaling"]
+                sc = (float(g["factor"]), float(g["original"]), float(g["fast"]), float(g["slow"]))
+            kv_from = int(mc["kv_from"]) if mc.get("kv_from") is not None else -1
+            if kv_from >= i or kv_from < -1:
+                raise ValueError(f"layer {i}: kv_from={kv_from} must name an earlier layer")
+            layers.append(LayerSpec(kind="latent", heads=heads, kv_heads=1, dim=dim, vdim=vdim, q_rank=int(mc["q_rank"]), kv_rank=int(mc["kv_rank"]),
+                                    rot_dim=int(mc["rot_dim"]), rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                                    rot_scaling=sc, scale=float(mc["scale"]), gated=True, kv_from=kv_from, **ff))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+    return LayerListConfig(family="Zefapel", width=int(config["width"]), vocab=int(config["vocab"]), norm_eps=float(config["norm"]["eps"]),
+                           residual_mult=1.0, layers=layers, norm_offset=0.0, norm_kind="dyt", block="sequential", layer_scale=True,
+                           embed_scale=float(config["embedding"]["scale"]))
+
+
+def _norm_shapes(cfg: LayerListConfig, name: str) -> dict[str, tuple[int, ...]]:
+    if cfg.norm_kind == "dyt":
+        return {name: (cfg.width,), name + ".b": (cfg.width,), name + ".alpha": ()}
+    return {name: (cfg.width,)}
+
+
+def _zefapel_tensor_shapes(cfg: LayerListConfig) -> dict[str, Any]:
+    """Every tensor a Zefapel checkpoint must hold, with its shape; a dimension of -1 is read from the file (the decay's rank)."""
+    W = cfg.width
+    want: dict[str, Any] = {"embed": (cfg.vocab, W), "head": (cfg.vocab, W), **_norm_shapes(cfg, "final.norm")}
+    for i, L in enumerate(cfg.layers):
+        p, m = cfg.prefix(i), cfg.prefix(i) + "mix."
+        want.update(_norm_shapes(cfg, p + "norm1"))
+        want[p + "ls1"] = (W,)
+        hv = L.heads * L.vdim
+        want.update({m + "g": (hv, W), m + "o": (W, hv)})
+        if L.kind == "linrec":
+            want.update({m + "q": (L.heads * L.dim, W), m + "k": (L.heads * L.dim, W), m + "v": (hv, W)})
+            if L.rec_kind == "expgate":
+                want.update({m + "i": (L.heads, W), m + "i.b": (L.heads,), m + "f": (L.heads, W), m + "f.b": (L.heads,), m + "norm": (hv,)})
+            else:
+                want.update({m + "a1": (L.a_rank, W), m + "a2": (L.heads * L.dim, L.a_rank), m + "a2.b": (L.heads * L.dim,), m + "norm": (L.vdim,)})
+        else:
+            want.update({m + "dq": (L.q_rank, W), m + "dq.norm": (L.q_rank,), m + "uq": (L.heads * (L.dim + L.rot_dim), L.q_rank),
+                         m + "uk": (L.heads * L.dim, L.kv_rank), m + "uv": (hv, L.kv_rank)})
+            if L.kv_from < 0:
+                want.update({m + "dkv": (L.kv_rank + L.rot_dim, W), m + "dkv.norm": (L.kv_rank,)})
+        if L.ff:
+            f = p + "mlp."
+            want.update(_norm_shapes(cfg, p + "norm2"))
+            want[p + "ls2"] = (W,)
+            if L.ff_kind == "gated":
+                want.update({f + "gate": (L.ff, W), f + "up": (L.ff, W), f + "down": (W, L.ff)})
+            else:
+                want.update({f + "router": (L.experts + L.identity, W), f + "correction": (L.experts + L.identity,)})
+                for e in range(L.experts):
+                    want.update({f + f"e{e}.up": (L.expert_ff, W), f + f"e{e}.down": (W, L.expert_ff)})
+                if L.shared_ff:
+                    want.update({f + "shared.up": (L.shared_ff, W), f + "shared.down": (W, L.shared_ff), f + "shared.sg": (1, W)})
+    return want
+
+
 # architecture name (config.json) -> (config reader, tensor table)
 FAMILIES: dict[str, tuple[Callable[[dict], LayerListConfig], Callable[[LayerListConfig], dict]]] = {
     "Fonapel": (fonapel_config, _fonapel_tensor_shapes),
+    "Zefapel": (zefapel_config, _zefapel_tensor_shapes),
 }
 
 
 def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtype: torch.dtype, device: Any) -> dict:
-    """The engine's weight layout from a family's named tensors: per layer one input matrix (every projection that reads
-    the normed input, rows concatenated: q | k | v | gate | [a | b] | up) and one output matrix ([W_o | W_down] side by
-    side); vectors in float32.  Matrices are cast to ``dtype`` (bfloat16 as stored, or float32)."""
+    """The engine's weight layout from a family's named tensors: per layer one input matrix (every projection that reads the
+    normed input, rows concatenated in the order include/tinyllm_hybrid.h lists per mixer kind) and one output matrix; in the
+    parallel block the feed-forward's rows / columns are appended to them, in the sequential block it has a pair of its own
+    (``w_in2`` / ``w_out2``).  Vectors in float32.  Matrices are cast to ``dtype`` (bfloat16 as stored, or float32)."""
     def mat(name):
         return tensors[name].to(device=device, dtype=dtype)
 
     def vec(name):
         return tensors[name].to(device=device, dtype=torch.float32).contiguous()
 
-    packed = {"embed": mat("embed").contiguous(), "head": mat("head").contiguous(), "final_norm": vec("final.norm"), "layers": []}
+    def norm(entry, key, name):
+        entry[key] = vec(name)
+        if cfg.norm_kind == "dyt":
+            entry[key + "_bias"], entry[key + "_alpha"] = vec(name + ".b"), float(tensors[name + ".alpha"].float())
+
+    packed: dict[str, Any] = {"embed": mat("embed").contiguous(), "head": mat("head").contiguous(), "layers": []}
+    norm(packed, "final_norm", "final.norm")
     if cfg.loop:
         packed["loop_in"] = mat("loop.in").contiguous()
         packed["loop_step"] = vec("loop.step")
     for i, L in enumerate(cfg.layers):
         p = cfg.prefix(i)
-        rows = [mat(p + "mix.q"), mat(p + "mix.k"), mat(p + "mix.v")]
-        if L.kind == "delta" or L.gated:
-            rows.append(mat(p + "mix.g"))
-        entry: dict[str, Any] = {"norm": vec(p + "norm1")}
+        entry: dict[str, Any] = {}
+        norm(entry, "norm", p + "norm1")
+        if L.kind == "latent":
+            rows = [mat(p + "mix.dq")] + ([mat(p + "mix.dkv")] if L.kv_from < 0 else []) + [mat(p + "mix.g")]
+            entry["dq_norm"], entry["uq"] = vec(p + "mix.dq.norm"), mat(p + "mix.uq").contiguous()
+            if L.kv_from < 0:
+                entry["dkv_norm"] = vec(p + "mix.dkv.norm")
+            # per head: W_uk transposed ([kv_rank, dim]: the key projection is applied to the query), W_uv as stored ([vdim, kv_rank])
+            entry["uk_t"] = mat(p + "mix.uk").reshape(L.heads, L.dim, L.kv_rank).transpose(1, 2).contiguous()
+            entry["uv"] = mat(p + "mix.uv").reshape(L.heads, L.vdim, L.kv_rank).contiguous()
+        else:
+            rows = [mat(p + "mix.q"), mat(p + "mix.k"), mat(p + "mix.v")]
+            if L.kind != "attention" or L.gated:
+                rows.append(mat(p + "mix.g"))
         if L.kind == "delta":
             rows += [mat(p + "mix.a"), mat(p + "mix.b")]
             entry["conv"] = torch.cat([vec(p + "mix.q.conv"), vec(p + "mix.k.conv"), vec(p + "mix.v.conv")], 0).contiguous()
             entry["a_log"], entry["dt_bias"], entry["out_norm"] = vec(p + "mix.A_log"), vec(p + "mix.dt_bias"), vec(p + "mix.norm")
+        elif L.kind == "linrec":
+            entry["out_norm"] = vec(p + "mix.norm")
+            if L.rec_kind == "expgate":
+                rows += [mat(p + "mix.i"), mat(p + "mix.f")]
+                entry["i_bias"], entry["f_bias"] = vec(p + "mix.i.b"), vec(p + "mix.f.b")
+            else:
+                rows.append(mat(p + "mix.a1"))
+                entry["a2"], entry["a2_bias"] = mat(p + "mix.a2").contiguous(), vec(p + "mix.a2.b")
         out = [mat(p + "mix.o")]
         if L.ff:
-            rows.append(mat(p + "mlp.up"))
-            out.append(mat(p + "mlp.down"))
+            f = p + "mlp."
+            if L.ff_kind == "plain":
+                ff_rows, ff_out = [mat(f + "up")], [mat(f + "down")]
+            elif L.ff_kind == "gated":
+                ff_rows, ff_out = [mat(f + "gate"), mat(f + "up")], [mat(f + "down")]
+            else:
+                W = cfg.width
+                shared = [mat(f + "shared.up")] if L.shared_ff else []
+                sg = mat(f + "shared.sg") if L.shared_ff else torch.zeros(1, W, device=device, dtype=dtype)
+                ff_rows = [mat(f + "router"), sg] + shared + [mat(f + f"e{e}.up") for e in range(L.experts)]
+                ff_out = ([mat(f + "shared.down")] if L.shared_ff else []) + [mat(f + f"e{e}.down") for e in range(L.experts)]
+                entry["correction"] = vec(f + "correction")
+            if cfg.block == "parallel":
+                rows, out = rows + ff_rows, out + ff_out
+            else:
+                norm(entry, "norm2", p + "norm2")
+                entry["w_in2"], entry["w_out2"] = torch.cat(ff_rows, 0).contiguous(), torch.cat(ff_out, 1).contiguous()
+        if cfg.layer_scale:
+            entry["ls1"] = vec(p + "ls1")
+            if L.ff:
+                entry["ls2"] = vec(p + "ls2")
         entry["w_in"] = torch.cat(rows, 0).contiguous()
         entry["w_out"] = torch.cat(out, 1).contiguous()
         packed["layers"].append(entry)

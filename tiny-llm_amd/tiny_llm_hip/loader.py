@@ -101,6 +101,9 @@ def _load_layer_list(model_dir: Path, config: dict, dtype: torch.dtype | None) -
     cfg = read_config(config)
     src = _TensorSource(model_dir)
     tensors = {}
+    for i, L in enumerate(cfg.layers):  # a size the configuration leaves to the tensors (the rank of a decay's projection pair)
+        if getattr(L, "a_rank", 0) < 0:
+            L.a_rank = int(src.get(cfg.prefix(i) + "mix.a1").shape[0])
     for name, shape in tensor_shapes(cfg).items():
         t = src.get(name)
         if tuple(t.shape) != tuple(shape):
