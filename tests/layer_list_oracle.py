@@ -380,3 +380,97 @@ def zefapel_forward(config, W, tokens, streams=None):
             streams.append(x.copy())
     xf = dyt_norm(x, W["final.norm.alpha"], W["final.norm"], W["final.norm.b"])
     return xf @ W["head"].T
+
+
+def make_zefapel_weights(config, seed=0):
+    """Random bf16-representable weights by tensor name (float32 arrays) for a Zefapel config dict."""
+    import torch
+
+    gen = torch.Generator().manual_seed(seed)
+    Wd, out = config["width"], {}
+
+    def mat(rows, cols, scale=None):
+        s = scale if scale is not None else cols ** -0.5
+        return (torch.randn(rows, cols, generator=gen) * s).to(torch.bfloat16).float().numpy()
+
+    def vec(n, scale=0.1, shift=0.0):
+        return (torch.randn(n, generator=gen) * scale + shift).to(torch.bfloat16).float().numpy()
+
+    def norm(name):
+        out[name], out[name + ".b"] = vec(Wd, 0.1, 1.0), vec(Wd, 0.05)
+        out[name + ".alpha"] = np.float32(vec(1, 0.1, 0.7)[0])
+
+    out["embed"], out["head"] = mat(config["vocab"], Wd, 1.0), mat(config["vocab"], Wd)
+    norm("final.norm")
+    for i, spec in enumerate(config["layers"]):
+        p, m, mc = f"l{i}.", f"l{i}.mix.", spec["mixer"]
+        H, D, V = mc["heads"], mc["dim"], mc["vdim"]
+        norm(p + "norm1")
+        out[p + "ls1"] = vec(Wd, 0.2, 0.8)
+        out[m + "g"], out[m + "o"] = mat(H * V, Wd), mat(Wd, H * V)
+        if spec["type"] in ("mlstm", "gla"):
+            out[m + "q"], out[m + "k"], out[m + "v"] = mat(H * D, Wd), mat(H * D, Wd), mat(H * V, Wd)
+            if spec["type"] == "mlstm":
+                out[m + "i"], out[m + "f"] = mat(H, Wd, 0.3), mat(H, Wd, 0.3)
+                out[m + "i.b"], out[m + "f.b"], out[m + "norm"] = vec(H, 1.0, -1.0), vec(H, 1.0, 3.0), vec(H * V, 0.1, 1.0)
+            else:
+                r = mc.get("a_rank", 6)
+                out[m + "a1"], out[m + "a2"], out[m + "a2.b"] = mat(r, Wd), mat(H * D, r), vec(H * D, 1.0, 1.0)
+                out[m + "norm"] = vec(V, 0.1, 1.0)
+        else:
+            Q, C, R = mc["q_rank"], mc["kv_rank"], mc["rot_dim"]
+            out[m + "dq"], out[m + "dq.norm"], out[m + "uq"] = mat(Q, Wd), vec(Q, 0.1, 1.0), mat(H * (D + R), Q)
+            out[m + "uk"], out[m + "uv"] = mat(H * D, C), mat(H * V, C)
+            if "kv_from" not in mc:
+                out[m + "dkv"], out[m + "dkv.norm"] = mat(C + R, Wd), vec(C, 0.1, 1.0)
+        mlp = spec.get("mlp")
+        if mlp:
+            f = p + "mlp."
+            norm(p + "norm2")
+            out[p + "ls2"] = vec(Wd, 0.2, 0.8)
+            if mlp["kind"] == "dense":
+                out[f + "gate"], out[f + "up"], out[f + "down"] = mat(mlp["ff"], Wd), mat(mlp["ff"], Wd), mat(Wd, mlp["ff"])
+            else:
+                r = mlp["router"]
+                ET = r["experts"] + r.get("identity", 0)
+                out[f + "router"], out[f + "correction"] = mat(ET, Wd, 2.0 * Wd ** -0.5), vec(ET, 0.1)
+                for e in range(r["experts"]):
+                    out[f + f"e{e}.up"], out[f + f"e{e}.down"] = mat(mlp["expert"]["ff"], Wd), mat(Wd, mlp["expert"]["ff"])
+                if mlp.get("shared"):
+                    s = mlp["shared"]["ff"]
+                    out[f + "shared.up"], out[f + "shared.down"], out[f + "shared.sg"] = mat(s, Wd), mat(Wd, s), mat(1, Wd)
+    return out
+
+
+def dense_ff(ff=72):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_ff(experts=5, identity=1, top=2, groups=3, keep=2, ff=24, shared=40):
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "identity": identity, "top": top, "groups": {"count": groups, "keep": keep}}}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+def mlstm_layer(heads=3, dim=24, vdim=16, gate_cap=12.0, mlp=None):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": gate_cap}, "mlp": mlp}
+
+
+def gla_layer(heads=2, dim=16, vdim=24, tau=8.0, a_rank=6, mlp=None):
+    """(a_rank is not a key of the checkpoint format: readers take it from the tensor; the weight maker reads it here)"""
+    return {"type": "gla", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "a_rank": a_rank}, "mlp": mlp}
+
+
+def latent_layer(heads=4, dim=16, vdim=24, rot_dim=8, q_rank=20, kv_rank=40, base=5000.0, scale=0.2, scaling=(4.0, 64, 16.0, 2.0), kv_from=None, mlp=None):
+    rot = {"base": base, "dims": rot_dim}
+    if scaling:
+        rot["scaling"] = {"factor": scaling[0], "original": scaling[1], "fast": scaling[2], "slow": scaling[3]}
+    mixer = {"heads": heads, "dim": dim, "vdim": vdim, "rot_dim": rot_dim, "q_rank": q_rank, "kv_rank": kv_rank, "rot": rot, "scale": scale}
+    if kv_from is not None:
+        mixer["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": mixer, "mlp": mlp}
+
+
+def zefapel_config(layers, width=64, vocab=101, eps=1e-5, embed_scale=0.7):
+    return {"architecture": "Zefapel", "embedding": {"scale": embed_scale}, "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
