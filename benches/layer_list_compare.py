@@ -7,6 +7,12 @@ its roofline is made of -- the bytes a decode step must stream (weights once + K
 multiply-adds of a prefill chunk -- and the fraction of 8 TB/s / 2.5 PFLOP/s (dense bf16) that the measured time amounts to.
 The two models differ where the designs differ: bf16 matrices against 4-bit ones (4 x the bytes per decode step), two of
 four mixers recurrent (no K/V to stream, a sequential recurrence in prefill), one fused in/out product pair per layer.
+
+`--layer-list-family Zefapel` measures the Zefapel family instead, beside its closest existing model -- Fonapel, on the same
+engine -- at equal width, head count, head width and matrix elements per layer: 4 layers (matrix memory + gated feed-forward,
+gated linear attention + mixture of experts, latent attention + gated feed-forward, latent attention on the third layer's cache
++ mixture of experts).  Its roofline counts what the design needs, not what the engine computes: the experts a token takes (not
+all of them), a latent cache row of kv_rank + rot_dim per token.
 """
 
 from __future__ import annotations
@@ -28,6 +34,57 @@ def fonapel_config(width: int, layers: int = 4, vocab: int = 32768) -> dict:
     order = [delta, attn, attn, delta]
     return {"architecture": "Fonapel", "layers": [order[i % 4] for i in range(layers)], "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": vocab,
             "width": width}
+
+
+def zefapel_config(width: int, vocab: int = 32768) -> dict:
+    """Head width 128 like the other two; the latent cache row is 192 + 64 wide; gated feed-forward of 2 W (three matrices: as many
+    elements as the 3 W two-matrix one beside it); 8 experts of W / 2 + 2 identity experts in 5 groups (3 kept), 2 taken, a shared one of W."""
+    heads = max(1, width // 128)
+    dense = {"kind": "dense", "ff": 2 * width}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 5, "keep": 3}},
+           "shared": {"ff": width}}
+    rot = {"base": 1e6, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    latent = {"heads": heads, "dim": 128, "vdim": 128, "rot_dim": 64, "q_rank": max(64, width // 2), "kv_rank": 192, "rot": rot, "scale": 192 ** -0.5}
+    layers = [{"type": "mlstm", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "gate_cap": 20.0}, "mlp": dense},
+              {"type": "gla", "mixer": {"heads": heads, "dim": 128, "vdim": 128, "tau": 8.0}, "mlp": moe},
+              {"type": "latent_attention", "mixer": dict(latent), "mlp": dense},
+              {"type": "latent_attention", "mixer": dict(latent, kv_from=2), "mlp": moe}]
+    return {"architecture": "Zefapel", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
+
+
+def zefapel_costs(cfg: dict, ctx: int, dtype_bytes: int = 2) -> dict:
+    """What the design needs: matrix elements a token multiplies (the experts it takes, not all), attention multiply-adds per
+    (query, key) pair in the per-head form, the bytes a decode step of b sequences must stream (every matrix once, but of the
+    experts only those b tokens can take; one latent row per cached token; the recurrent states read and written)."""
+    W, fixed, per_expert, experts_taken, kv_per_tok, state, attn = cfg["width"], 0, [], [], 0, 0, 0
+    for L in cfg["layers"]:
+        m, mlp = L["mixer"], L["mlp"]
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        if L["type"] == "mlstm":
+            fixed += W * (2 * H * D + 2 * H * V + 2 * H) + H * V * W
+            state += H * D * (V + 1)
+        elif L["type"] == "gla":
+            fixed += W * (2 * H * D + 2 * H * V + 16) + 16 * H * D + H * V * W  # (synthetic weights: a decay projection pair of rank 16)
+            state += H * D * V
+        else:
+            R, C, Q = m["rot_dim"], m["kv_rank"], m["q_rank"]
+            fixed += W * Q + Q * H * (D + R) + H * (D + V) * C + 2 * H * V * W
+            if "kv_from" not in m:
+                fixed += W * (C + R)
+                kv_per_tok += C + R
+            attn += H * (D + R + V)
+        if mlp and mlp["kind"] == "dense":
+            fixed += 3 * W * mlp["ff"]
+        elif mlp:
+            r = mlp["router"]
+            fixed += W * (r["experts"] + r.get("identity", 0)) + (2 * W * mlp["shared"]["ff"] + W if mlp.get("shared") else 0)
+            per_expert.append(2 * W * mlp["expert"]["ff"])
+            experts_taken.append((r["top"], r["experts"]))
+    head = cfg["vocab"] * W
+    active = fixed + sum(pe * top for pe, (top, _) in zip(per_expert, experts_taken))
+    return {"matrix_elems": active, "head_elems": head, "attn_macs_per_pair": attn,
+            "decode_bytes": lambda b: (fixed + head + sum(pe * min(n, b * top) for pe, (top, n) in zip(per_expert, experts_taken))) * dtype_bytes
+            + b * (ctx * kv_per_tok * dtype_bytes + 2 * state * 4)}
 
 
 def qwen3_config(width: int, layers: int = 4, vocab: int = 32768) -> dict:
@@ -105,6 +162,39 @@ def measure(engine, prompt, decode_steps: int, batches=(1, 4), free_running=None
     return out
 
 
+def run_family_pair(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, device: str = "cuda") -> dict:
+    """Zefapel beside Fonapel, both on the layer-list engine."""
+    import torch
+
+    from tiny_llm_hip.models import engine_for
+    from tiny_llm_hip.synthetic import synthetic_layer_list
+
+    rng = random.Random(seed)
+    results = []
+    for W in widths:
+        prompt = [rng.randrange(1, 32768) for _ in range(prompt_len)]
+        ctx = prompt_len + decode_steps
+        page = 128
+        pages = 4 * ((prompt_len + 3 * decode_steps) // page + 2)
+        row = {"width": W, "prompt_len": prompt_len, "decode_steps": decode_steps}
+        for key, cfg, costs in (("zefapel", zefapel_config(W), zefapel_costs), ("fonapel", fonapel_config(W), fonapel_costs)):
+            model = synthetic_layer_list(cfg, seed=seed, device=device)
+            eng = engine_for(model, dtype=torch.bfloat16, page_size=page, num_pages=pages, max_batch=4, max_pages_per_seq=pages // 4, max_prefill_rows=prompt_len)
+            try:
+                got = measure(eng, prompt, decode_steps, free_running=eng.decode_free_running)
+            finally:
+                eng.close()
+            del model
+            row[key] = summarize(got, costs(cfg, ctx), prompt_len)
+            torch.cuda.empty_cache()
+        for leg in ("prefill", "decode_b1", "decode_b4"):
+            a, b = row["zefapel"][leg]["roofline_fraction"], row["fonapel"][leg]["roofline_fraction"]
+            row.setdefault("times_as_far_from_roofline", {})[leg] = round(b / a, 2) if a > 0 else None
+        results.append(row)
+    return {"bench": "layer_list_compare", "family": "Zefapel", "beside": "Fonapel", "dtype": "bf16", "data": "synthetic",
+            "roofline": {"hbm_bytes_per_s": HBM_BYTES_PER_S, "bf16_flops": BF16_FLOPS}, "results": results}
+
+
 def run(widths, prompt_len: int = 2048, decode_steps: int = 64, seed: int = 0, device: str = "cuda") -> dict:
     import torch
 
@@ -162,5 +252,7 @@ def summarize(got: dict, costs: dict, prompt_len: int) -> dict:
     return out
 
 
-def main(widths, prompt_len=2048, decode_steps=64) -> None:
-    print(json.dumps(run(widths, prompt_len, decode_steps)), flush=True)
+def main(widths, prompt_len=2048, decode_steps=64, family="Fonapel") -> None:
+    if family not in ("Fonapel", "Zefapel"):
+        raise SystemExit(f"--layer-list-family: unknown family {family!r}")
+    print(json.dumps((run if family == "Fonapel" else run_family_pair)(widths, prompt_len, decode_steps)), flush=True)

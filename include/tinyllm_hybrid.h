@@ -85,8 +85,8 @@ enum { TL_HY_F32 = 0, TL_HY_BF16 = 2 }; /* the values of tl_dtype in tinyllm_hip
  *   norm2 through w_in2 and returns through w_out2:
  *   plain: up (ff)                   -> w_out2 [width, ff]
  *   gated: gate (ff) | up (ff)       -> w_out2 [width, ff]
- *   moe:   router (experts + identity) | shared gate (1) | shared up (shared_ff) | expert 0 up (expert_ff) | expert 1 up ...
- *                                    -> w_out2 [width, shared_ff + experts * expert_ff]: shared down | expert 0 down | ... */
+ *   moe:   shared up (shared_ff) | expert 0 up (expert_ff) | expert 1 up ... | router (experts + identity) | shared gate (1) |
+ *          zero rows up to a multiple of 8         -> w_out2 [width, shared_ff + experts * expert_ff]: shared down | expert 0 down | ... */
 typedef struct tl_hybrid_layer {
     int kind;
     int heads, kv_heads, dim, vdim;

@@ -107,7 +107,7 @@ static int mixer_cols(const tl_hybrid_layer &L) {  // rows of w_in that belong t
 static int ff_in_cols(const tl_hybrid_layer &L) {  // rows of the feed-forward's input matrix
     if (L.ff <= 0) return 0;
     if (L.ff_kind == TL_FF_GATED) return 2 * L.ff;
-    if (L.ff_kind == TL_FF_MOE) return L.experts + L.identity + 1 + L.shared_ff + L.experts * L.expert_ff;
+    if (L.ff_kind == TL_FF_MOE) return (L.shared_ff + L.experts * L.expert_ff + L.experts + L.identity + 1 + 7) / 8 * 8;
     return L.ff;
 }
 static int conv_channels(const tl_hybrid_layer &L) { return 2 * L.kv_heads * L.dim + L.heads * L.vdim; }
@@ -436,8 +436,8 @@ static int ff_act_t(tl_hybrid *e, const tl_hybrid_layer &L, int rows, int ldp, i
     using S = typename D::storage;
     hipStream_t st = e->stream;
     if (L.ff_kind == TL_FF_MOE) {
-        const int ET = L.experts + L.identity;
-        hipLaunchKernelGGL((moe_route_act_kernel<D>), dim3(rows), dim3(256), 0, st, e->proj, ldp, up0, up0 + ET, up0 + ET + 1, up0 + ET + 1 + L.shared_ff,
+        const int ET = L.experts + L.identity, r0 = up0 + L.ff;  // shared up | expert ups | router | shared gate | padding
+        hipLaunchKernelGGL((moe_route_act_kernel<D>), dim3(rows), dim3(256), 0, st, e->proj, ldp, r0, r0 + ET, up0, up0 + L.shared_ff,
                            L.experts, L.identity, L.top, L.groups, L.keep, L.expert_ff, L.shared_ff, L.correction_dev, (S *)e->cat, ldcat, col0, e->idw);
         TL_CHECK_LAUNCH("hybrid moe route");
         return TL_OK;

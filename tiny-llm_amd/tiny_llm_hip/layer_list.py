@@ -332,7 +332,10 @@ def pack_layer_list(cfg: LayerListConfig, tensors: dict[str, torch.Tensor], dtyp
                 W = cfg.width
                 shared = [mat(f + "shared.up")] if L.shared_ff else []
                 sg = mat(f + "shared.sg") if L.shared_ff else torch.zeros(1, W, device=device, dtype=dtype)
-                ff_rows = [mat(f + "router"), sg] + shared + [mat(f + f"e{e}.up") for e in range(L.experts)]
+                ff_rows = shared + [mat(f + f"e{e}.up") for e in range(L.experts)] + [mat(f + "router"), sg]
+                pad = -sum(r.shape[0] for r in ff_rows) % 8  # the engine's row count of this matrix is a multiple of 8
+                if pad:
+                    ff_rows.append(torch.zeros(pad, W, device=device, dtype=dtype))
                 ff_out = ([mat(f + "shared.down")] if L.shared_ff else []) + [mat(f + f"e{e}.down") for e in range(L.experts)]
                 entry["correction"] = vec(f + "correction")
             if cfg.block == "parallel":

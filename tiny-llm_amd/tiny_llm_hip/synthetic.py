@@ -136,16 +136,21 @@ def synthetic_layer_list(config: dict, seed: int = 0, device: str = "cuda", dtyp
     gen = torch.Generator(device=device)
     gen.manual_seed(seed)
     tensors = {}
+    for i, L in enumerate(cfg.layers):  # a size the checkpoint format leaves to the tensors
+        if getattr(L, "a_rank", 0) < 0:
+            L.a_rank = 16
+    # vectors that multiply (norm weights applied as they are, layer scales) are drawn around 1, biases that open a gate around their shift
+    around_one = ("mix.norm", ".alpha") + ((".norm1", ".norm2", "final.norm", "dq.norm", "dkv.norm", ".ls1", ".ls2") if cfg.norm_offset == 0.0 else ())
+    shifts = {"mix.f.b": 3.0, "mix.a2.b": 2.0}
     for name, shape in tensor_shapes(cfg).items():
+        shift = 1.0 if name.endswith(around_one) else next((v for k, v in shifts.items() if name.endswith(k)), 0.0)
         if len(shape) == 2 and not name.endswith(".conv") and name != "loop.step":
             scale = 1.0 if name == "embed" else shape[1] ** -0.5
-        elif name.endswith("mix.norm"):
+        elif name.endswith("mix.norm") or name.endswith(".alpha"):
             scale = 0.0
         else:
-            scale = 0.1 if len(shape) == 1 else 0.5
-        t = torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * scale
-        if name.endswith("mix.norm"):
-            t = t + 1.0
+            scale = 0.1 if len(shape) <= 1 else 0.5
+        t = torch.randn(tuple(shape), generator=gen, device=device, dtype=torch.float32) * scale + shift
         tensors[name] = t.to(torch.bfloat16)
     args = SimpleNamespace(vocab_size=cfg.vocab, hidden_size=cfg.width, num_hidden_layers=len(cfg.layers), architecture=cfg.family)
     return SimpleNamespace(family=cfg.family, config=cfg, tensors=tensors, dtype=dtype, args=args)
