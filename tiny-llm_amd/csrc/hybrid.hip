@@ -302,6 +302,7 @@ static int attention_core(tl_hybrid *e, const tl_hybrid_layer &L, const void *kp
     }
     if (dk4 <= 16 && vt_n <= 4) return launch_attn_tile<D, 16, 4>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
     if (dk4 <= 32 && vt_n <= 8) return launch_attn_tile<D, 32, 8>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
+    if (vt_n <= 12) return launch_attn_tile<D, 64, 12>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);  // (a 192-wide latent beside a 64-wide rotated part)
     return launch_attn_tile<D, 64, 16>(e, L, kpool, vpool, v_row, m, sh, gate, ldg, out, ldo);
 }
 
@@ -310,8 +311,9 @@ static int launch_linrec(const tl_hybrid *e, const tl_hybrid_layer &L, const Run
     const int ones = chan ? 0 : 1, VE = L.vdim + ones;
     // lanes per state column: a wave while the step's columns are few (decode), a DPP row of 16 otherwise (or for narrow keys)
     const long cols = (long)L.heads * VE * n_seqs, simds = 4 * (long)qmm3_num_cus();
-    int lpc = (cols <= simds && L.dim > 16) ? 64 : 16;
-    if (L.dim > 16 * 16) lpc = 64;
+    int lpc = cols <= simds ? 64 : (cols <= 2 * simds + simds / 8 ? 32 : 16);
+    while (lpc > 16 && lpc >= 2 * L.dim) lpc /= 2;  // no more lanes than key rows
+    while (lpc < 64 && lpc * 16 < L.dim) lpc *= 2;  // at most 16 rows a lane
     int rpt = 1;
     while (lpc * rpt < L.dim) rpt *= 2;
     TL_REQUIRE(rpt <= 16, "hybrid linrec: key width above 1024 is not supported");
@@ -330,6 +332,8 @@ static int launch_linrec(const tl_hybrid *e, const tl_hybrid_layer &L, const Run
     }
     if (lpc == 64) {
         if (chan) { HY_LR_R(64, true) } else { HY_LR_R(64, false) }
+    } else if (lpc == 32) {
+        if (chan) { HY_LR_R(32, true) } else { HY_LR_R(32, false) }
     } else {
         if (chan) { HY_LR_R(16, true) } else { HY_LR_R(16, false) }
     }
@@ -437,7 +441,7 @@ static int ff_act_t(tl_hybrid *e, const tl_hybrid_layer &L, int rows, int ldp, i
     hipStream_t st = e->stream;
     if (L.ff_kind == TL_FF_MOE) {
         const int ET = L.experts + L.identity, r0 = up0 + L.ff;  // shared up | expert ups | router | shared gate | padding
-        hipLaunchKernelGGL((moe_route_act_kernel<D>), dim3(rows), dim3(256), 0, st, e->proj, ldp, r0, r0 + ET, up0, up0 + L.shared_ff,
+        hipLaunchKernelGGL((moe_route_act_kernel<D>), dim3(rows, rows >= 64 ? 1 : std::max(1, std::min(64, L.ff / 1024))), dim3(256), 0, st, e->proj, ldp, r0, r0 + ET, up0, up0 + L.shared_ff,
                            L.experts, L.identity, L.top, L.groups, L.keep, L.expert_ff, L.shared_ff, L.correction_dev, (S *)e->cat, ldcat, col0, e->idw);
         TL_CHECK_LAUNCH("hybrid moe route");
         return TL_OK;

@@ -1036,7 +1036,8 @@ __global__ __launch_bounds__(256) void linrec_kernel(const float *proj, int ldp,
                                                      int vdim, int ones) {
     constexpr int DP = LPC * RPT, CPB = 256 / LPC;
     constexpr int TB = 4096 / DP < 32 ? 4096 / DP : 32;
-    __shared__ float qs[TB * DP], ks[TB * DP], as[CHAN ? TB * DP : TB], vs[TB * CPB], bs[TB], os[TB * CPB];
+    __shared__ __attribute__((aligned(16))) float qs[TB * DP], ks[TB * DP], as[CHAN ? TB * DP : TB];
+    __shared__ float vs[TB * CPB], bs[TB], os[TB * CPB];
     const int h = blockIdx.x, s = blockIdx.y, j0 = blockIdx.z * CPB, VE = vdim + ones;
     const int r0 = seq_row0[s], n = seq_row0[s + 1] - r0, slot = seq_slot[s];
     const int tid = threadIdx.x, jl = tid / LPC, r = tid % LPC, j = j0 + jl;
@@ -1045,43 +1046,94 @@ __global__ __launch_bounds__(256) void linrec_kernel(const float *proj, int ldp,
     float *sp = state + (((size_t)slot * H + h) * VE + (active ? j : 0)) * dim + r * RPT;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) S[i] = (active && r * RPT + i < dim) ? sp[i] : 0.f;
+    // The next tile's inputs travel through registers: loaded before the current tile's recurrence starts, written to LDS after it, so the
+    // loads' latency hides behind the token loop (as in delta_kernel).
+    constexpr int NIT = TB * DP / 256, NV = (TB * CPB + 255) / 256;
+    float rq[NIT], rk[NIT], ra[CHAN ? NIT : 1], rv[NV], rg = 1.f, rb = 0.f;
+    auto fetch = [&](int t0) __attribute__((always_inline)) {
+        const int nt = min(TB, n - t0);
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int i = tid + 256 * it, tt = i / DP, d = i % DP;
+            const bool ok = tt < nt && d < dim;
+            const float *row = proj + (size_t)(r0 + t0 + (ok ? tt : 0)) * ldp + (size_t)h * dim + (ok ? d : 0);
+            rq[it] = ok ? row[q0] : 0.f;
+            rk[it] = ok ? row[k0] : 0.f;
+            if constexpr (CHAN) ra[it] = ok ? decay[((size_t)(r0 + t0 + tt) * H + h) * dim + d] : 1.f;
+        }
+#pragma unroll
+        for (int it = 0; it < NV; ++it) {
+            const int i = tid + 256 * it, tt = i / CPB, c = j0 + i % CPB;
+            rv[it] = (tt < nt && c < VE) ? (c < vdim ? proj[(size_t)(r0 + t0 + tt) * ldp + v0 + (size_t)h * vdim + c] : 1.f) : 0.f;
+        }
+        if (tid < nt) {
+            if constexpr (!CHAN) rg = gates[((size_t)(r0 + t0 + tid) * H + h) * 3];
+            rb = CHAN ? 1.f : gates[((size_t)(r0 + t0 + tid) * H + h) * 3 + 1];
+        }
+    };
+    if (n > 0) fetch(0);
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int nt = min(TB, n - t0);
-        __syncthreads();
-        for (int i = tid; i < TB * DP; i += 256) {
-            const int tt = i / DP, d = i % DP;
-            const bool ok = tt < nt && d < dim;
-            const float *row = proj + (size_t)(r0 + t0 + (ok ? tt : 0)) * ldp + (size_t)h * dim + d;
-            qs[i] = ok ? row[q0] : 0.f;
-            ks[i] = ok ? row[k0] : 0.f;
-            if constexpr (CHAN) as[i] = ok ? decay[((size_t)(r0 + t0 + tt) * H + h) * dim + d] : 1.f;
+        __syncthreads();  // the previous tile's recurrence is done with the LDS
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            qs[tid + 256 * it] = rq[it];
+            ks[tid + 256 * it] = rk[it];
+            if constexpr (CHAN) as[tid + 256 * it] = ra[it];
         }
-        for (int i = tid; i < TB * CPB; i += 256) {
-            const int tt = i / CPB, c = j0 + i % CPB;
-            vs[i] = (tt < nt && c < VE) ? (c < vdim ? proj[(size_t)(r0 + t0 + tt) * ldp + v0 + (size_t)h * vdim + c] : 1.f) : 0.f;
-        }
+#pragma unroll
+        for (int it = 0; it < NV; ++it)
+            if (tid + 256 * it < TB * CPB) vs[tid + 256 * it] = rv[it];
         if (tid < TB) {
-            const bool ok = tid < nt;
-            if constexpr (!CHAN) as[tid] = ok ? gates[((size_t)(r0 + t0 + tid) * H + h) * 3] : 1.f;
-            bs[tid] = ok ? (CHAN ? 1.f : gates[((size_t)(r0 + t0 + tid) * H + h) * 3 + 1]) : 0.f;
+            if constexpr (!CHAN) as[tid] = rg;
+            bs[tid] = rb;
         }
         __syncthreads();
+        if (t0 + TB < n) fetch(t0 + TB);
+        // the state's chain is one multiply-add per token and element; the next token's operands are read from LDS while the current one runs
+        float bv, kv[RPT], qv[RPT], av[CHAN ? RPT : 1];
+        auto read_token = [&](int tt, float &bv_, float (&k_)[RPT], float (&q_)[RPT], float (&a_)[CHAN ? RPT : 1]) __attribute__((always_inline)) {
+            bv_ = bs[tt] * vs[tt * CPB + jl];
+            const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT, *at = as + (CHAN ? tt * DP + r * RPT : tt);
+            if constexpr (RPT % 4 == 0) {
+#pragma unroll
+                for (int i = 0; i < RPT; i += 4) {
+                    const f32x4 k4 = *reinterpret_cast<const f32x4 *>(kt + i), q4 = *reinterpret_cast<const f32x4 *>(qt + i);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) k_[i + e] = k4[e], q_[i + e] = q4[e];
+                    if constexpr (CHAN) {
+                        const f32x4 a4 = *reinterpret_cast<const f32x4 *>(at + i);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) a_[i + e] = a4[e];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RPT; ++i) {
+                    k_[i] = kt[i], q_[i] = qt[i];
+                    if constexpr (CHAN) a_[i] = at[i];
+                }
+            }
+            if constexpr (!CHAN) a_[0] = at[0];
+        };
+        read_token(0, bv, kv, qv, av);
         for (int tt = 0; tt < nt; ++tt) {
-            const float bv = bs[tt] * vs[tt * CPB + jl];
-            const float *kt = ks + tt * DP + r * RPT, *qt = qs + tt * DP + r * RPT;
-            float a_s = 1.f;
-            if constexpr (!CHAN) a_s = as[tt];
+            float nbv, nk[RPT], nq[RPT], na[CHAN ? RPT : 1];
+            read_token(tt + 1 < nt ? tt + 1 : tt, nbv, nk, nq, na);
             float od0 = 0.f, od1 = 0.f;
 #pragma unroll
             for (int i = 0; i < RPT; ++i) {
-                float a = a_s;
-                if constexpr (CHAN) a = as[tt * DP + r * RPT + i];
-                S[i] = S[i] * a + kt[i] * bv;
-                if (i & 1) od1 += S[i] * qt[i];
-                else od0 += S[i] * qt[i];
+                S[i] = S[i] * av[CHAN ? i : 0] + kv[i] * bv;
+                if (i & 1) od1 += S[i] * qv[i];
+                else od0 += S[i] * qv[i];
             }
             const float od = column_sum<LPC>(od0 + od1, tid);
             if (r == 0) os[tt * CPB + jl] = od;
+            bv = nbv;
+#pragma unroll
+            for (int i = 0; i < RPT; ++i) kv[i] = nk[i], qv[i] = nq[i];
+#pragma unroll
+            for (int i = 0; i < (CHAN ? RPT : 1); ++i) av[i] = na[i];
         }
         __syncthreads();
         for (int i = tid; i < nt * CPB; i += 256) {
@@ -1120,8 +1172,8 @@ __global__ __launch_bounds__(64) void linrec_out_kernel(const float *obuf, int V
 }
 
 // ---- mixture of experts: routing and activation, one workgroup per row -----------------------------------------------------------------
-// proj columns of the row: router logits z [ET] at r0 (ET = experts + identity experts) | shared gate (1) at sg0 | shared up [ffs] at su0 |
-// expert e's up [ffe] at eu0 + e * ffe.  s = softmax(z); choice = s + correction; the experts form `groups` equal runs of neighbours, a
+// proj columns of the row: shared up [ffs] at su0, directly behind it expert e's up [ffe] at eu0 + e * ffe (eu0 = su0 + ffs); router logits
+// z [ET] at r0 (ET = experts + identity experts); shared gate (1) at sg0.  s = softmax(z); choice = s + correction; the experts form `groups` equal runs of neighbours, a
 // group scores its largest choice, only the `keep` best groups can be taken; the `top` largest choices among them are taken (ties: the lower
 // index); weights are their s, not renormalised.  The last `identity` experts return their input: their weights are summed into idw[t].
 // cat row: [ sigmoid(sg) * relu(up)^2  (ffs) | w_e * relu(up_e)^2 (ffe each; 0 for experts not taken) ].
@@ -1131,6 +1183,7 @@ __global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, i
                                                             typename D::storage *out, int ldo, int col0, float *idw) {
     __shared__ float sw[256], sc[256];
     __shared__ float gm[256];
+    // blockIdx.y: a share of the row's columns (every share routes the row again: a few dozen comparisons against thousands of columns)
     const int t = blockIdx.x, tid = threadIdx.x, ET = experts + identity;
     const float *row = proj + (size_t)t * ldp;
     if (tid < 64) {  // one wave routes (ET <= 256: four experts a lane at most)
@@ -1176,33 +1229,26 @@ __global__ __launch_bounds__(256) void moe_route_act_kernel(const float *proj, i
     }
     __syncthreads();
     float wgt = 0.f;
-    bool dead = true;
     if (tid < ET) {
         const float c = sc[tid];
-        dead = c == -INFINITY && true;
         int rank = 0;
         for (int o = 0; o < ET; ++o) rank += (sc[o] > c) || (sc[o] == c && o < tid);
         wgt = (rank < top && !(c == -INFINITY)) ? sw[tid] : 0.f;
     }
-    (void)dead;
     __syncthreads();
     if (tid < ET) sw[tid] = wgt;
     __syncthreads();
-    if (tid == 0) {
+    if (tid == 0 && blockIdx.y == 0) {
         float a = 0.f;
         for (int e = experts; e < ET; ++e) a += sw[e];
         idw[t] = a;
     }
     const float sgate = ffs > 0 ? sigmoid_f(row[sg0]) : 0.f;
     typename D::storage *o = out + (size_t)t * ldo + col0;
-    for (int c = tid; c < ffs; c += 256) {
-        const float u = fmaxf(row[su0 + c], 0.f);
-        o[c] = D::from_float(sgate * u * u);
-    }
-    const int n = experts * ffe;
-    for (int c = tid; c < n; c += 256) {
-        const float w = sw[c / ffe], u = fmaxf(row[eu0 + c], 0.f);
-        o[ffs + c] = D::from_float(w * u * u);
+    const int n = ffs + experts * ffe, per = (n + gridDim.y - 1) / gridDim.y, c_end = min(n, (int)(blockIdx.y + 1) * per);
+    for (int c = blockIdx.y * per + tid; c < c_end; c += 256) {  // shared columns first, then the experts' (su0 + ffs == eu0)
+        const float w = c < ffs ? sgate : sw[(c - ffs) / ffe], u = fmaxf(row[su0 + c], 0.f);
+        o[c] = D::from_float(w * u * u);
     }
 }
 // identity experts: x[t, c] += ls[c] * idw[t] * h[t, c]  (ls may be null: 1)
