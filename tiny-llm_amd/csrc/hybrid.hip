@@ -347,7 +347,8 @@ template <typename D>
 static int norm_t(tl_hybrid *e, int kind, const float *w, const float *b, float alpha, float offset, void *out, const int32_t *rows_idx, int rows) {
     using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
-    if (kind == TL_NORM_DYT) hipLaunchKernelGGL((dyt_kernel<D>), dim3(rows), dim3(256), 0, e->stream, e->x, w, b, alpha, (S *)out, c.width, rows_idx);
+    // (a few rows: more threads per row, one pass of loads in flight instead of several in a row)
+    if (kind == TL_NORM_DYT) hipLaunchKernelGGL((dyt_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, e->stream, e->x, w, b, alpha, (S *)out, c.width, rows_idx);
     else hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(256), 0, e->stream, e->x, w, offset, c.norm_eps, (S *)out, c.width, rows_idx);
     TL_CHECK_LAUNCH("hybrid norm");
     return TL_OK;
@@ -374,7 +375,7 @@ static int mixer_t(tl_hybrid *e, size_t ri, const Meta &m, const StepShape &sh, 
     if (L.kind == TL_MIX_LATENT) {
         // proj: dq (q_rank) | [dkv (kv_rank + rot_dim)] | gate (H * vdim)
         const int own = L.kv_from < 0, kv0 = L.q_rank, g0 = L.q_rank + (own ? L.kv_rank + L.rot_dim : 0), DT = L.kv_rank + L.rot_dim, DQ = L.dim + L.rot_dim;
-        hipLaunchKernelGGL((rms_cols_kernel<D>), dim3(rows), dim3(64), 0, st, e->proj, ldp, L.q_rank, L.dq_norm_dev, c.norm_eps, (S *)e->da, L.q_rank);
+        hipLaunchKernelGGL((rms_cols_kernel<D>), dim3(rows), dim3(rows < 64 ? 512 : 128), 0, st, e->proj, ldp, L.q_rank, L.dq_norm_dev, c.norm_eps, (S *)e->da, L.q_rank);
         TL_CHECK_LAUNCH("hybrid latent query norm");
         HY_TRY(linear_t<D>(e->da, L.q_rank, L.uq_dev, e->f32a, H * DQ, rows, H * DQ, L.q_rank, 0, 1.f, nullptr, 0, st));
         hipLaunchKernelGGL((latent_prep_kernel<D>), dim3(rows, H + 1), dim3(64), 0, st, e->f32a, H, L.dim, L.rot_dim, L.kv_rank, e->proj, ldp, kv0,

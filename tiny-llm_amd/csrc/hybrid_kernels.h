@@ -880,16 +880,17 @@ __global__ void dyt_kernel(const float *x, const float *w, const float *b, float
     for (int c = threadIdx.x; c < width; c += blockDim.x) out[(size_t)r * width + c] = D::from_float(tanhf(alpha * src[c]) * w[c] + b[c]);
 }
 
-// ---- RMS norm of n columns of float32 rows (a latent) -> D rows: x / sqrt(mean x^2 + eps) * w.  One wave per row. ----------------
+// ---- RMS norm of n columns of float32 rows (a latent) -> D rows: x / sqrt(mean x^2 + eps) * w.  One workgroup per row. -------------
 template <typename D>
-__global__ __launch_bounds__(64) void rms_cols_kernel(const float *in, int ldi, int n, const float *w, float eps, typename D::storage *out, int ldo) {
-    const int t = blockIdx.x, lane = threadIdx.x;
+__global__ void rms_cols_kernel(const float *in, int ldi, int n, const float *w, float eps, typename D::storage *out, int ldo) {
+    __shared__ float red[16];
+    const int t = blockIdx.x;
     const float *src = in + (size_t)t * ldi;
     float ss = 0.f;
-    for (int c = lane; c < n; c += 64) ss += src[c] * src[c];
-    ss = wave_sum(ss);
+    for (int c = threadIdx.x; c < n; c += blockDim.x) ss += src[c] * src[c];
+    ss = block_sum(ss, red);
     const float inv = 1.f / sqrtf(ss / (float)n + eps);
-    for (int c = lane; c < n; c += 64) out[(size_t)t * ldo + c] = D::from_float(src[c] * inv * w[c]);
+    for (int c = threadIdx.x; c < n; c += blockDim.x) out[(size_t)t * ldo + c] = D::from_float(src[c] * inv * w[c]);
 }
 
 // ---- latent attention, step 1.  Queries q [rows, H, dim + rot] (float32): the plain part -> qn (D, the input of the per-head key
