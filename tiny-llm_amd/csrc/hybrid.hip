@@ -349,7 +349,7 @@ static int norm_t(tl_hybrid *e, int kind, const float *w, const float *b, float 
     const tl_hybrid_config &c = e->cfg;
     // (a few rows: more threads per row, one pass of loads in flight instead of several in a row)
     if (kind == TL_NORM_DYT) hipLaunchKernelGGL((dyt_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, e->stream, e->x, w, b, alpha, (S *)out, c.width, rows_idx);
-    else hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(256), 0, e->stream, e->x, w, offset, c.norm_eps, (S *)out, c.width, rows_idx);
+    else hipLaunchKernelGGL((norm_kernel<D>), dim3(rows), dim3(rows < 64 ? 1024 : 256), 0, e->stream, e->x, w, offset, c.norm_eps, (S *)out, c.width, rows_idx);
     TL_CHECK_LAUNCH("hybrid norm");
     return TL_OK;
 }
