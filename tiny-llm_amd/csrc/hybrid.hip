@@ -144,10 +144,18 @@ static Meta carve(int32_t *base, int R, int S) {
 }
 static size_t meta_ints(int R, int S) { return (size_t)5 * R + 2 * S + 2; }
 
+// a Dynamic Tanh norm that may leave with the product completing a residual sum (epilogue 4 of the row and 64-wide tile kernels)
+struct NormTail {
+    const float *w = nullptr, *b = nullptr;
+    float alpha = 0.f;
+    void *out = nullptr;   // D rows of N
+    bool done = false;     // set by linear_t when the product carried it
+};
+
 // out (+)= A . W^T by shape: a few rows stream the weights once per column (row kernel), more go through the MFMA tile kernel
 template <typename D>
 static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, int M, int N, int K, int epi, float alpha, const float *bias,
-                    int force, hipStream_t st, int batch = 1, long sa = 0, long sw = 0, long sc = 0) {
+                    int force, hipStream_t st, int batch = 1, long sa = 0, long sw = 0, long sc = 0, NormTail *tail = nullptr) {
     using S = typename D::storage;
     if (M <= 0 || N <= 0 || batch <= 0) return TL_OK;
     const int vec_ok = (K % 8 == 0) && (lda % 8 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && sa % 8 == 0 && sw % 8 == 0;
@@ -172,21 +180,29 @@ static int linear_t(const void *A, int lda, const void *W, float *out, int ldc, 
         }
         TL_REQUIRE(force != 3, "hybrid linear: the 256-wide tile GEMM does not take this shape");
     }
-#define HY_GEMM(KERN, E) hipLaunchKernelGGL((KERN<D, E>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok, sa, sw, sc)
+    const bool with_tail = tail && tail->out && epi == 3 && batch == 1 && ldc == N;
+    const float *nw = with_tail ? tail->w : nullptr, *nb = with_tail ? tail->b : nullptr;
+    const float nalpha = with_tail ? tail->alpha : 0.f;
+    S *nout = with_tail ? (S *)tail->out : nullptr;
+#define HY_GEMM(KERN, E) \
+    hipLaunchKernelGGL((KERN<D, E>), grid, block, 0, st, (const S *)A, lda, (const S *)W, out, ldc, M, N, K, alpha, bias, vec_ok, sa, sw, sc, nw, nb, nalpha, nout)
     if (rows) {
         dim3 grid((N + 3) / 4, batch), block(256);
         if (epi == 0) HY_GEMM(gemm_rows_kernel, 0);
         else if (epi == 1) HY_GEMM(gemm_rows_kernel, 1);
         else if (epi == 2) HY_GEMM(gemm_rows_kernel, 2);
-        else HY_GEMM(gemm_rows_kernel, 3);
+        else if (!with_tail) HY_GEMM(gemm_rows_kernel, 3);
+        else HY_GEMM(gemm_rows_kernel, 4);
     } else {
         dim3 grid(((M + 63) / 64) * ((N + 63) / 64), batch), block(256);
         if (epi == 0) HY_GEMM(gemm_tile_kernel, 0);
         else if (epi == 1) HY_GEMM(gemm_tile_kernel, 1);
         else if (epi == 2) HY_GEMM(gemm_tile_kernel, 2);
-        else HY_GEMM(gemm_tile_kernel, 3);
+        else if (!with_tail) HY_GEMM(gemm_tile_kernel, 3);
+        else HY_GEMM(gemm_tile_kernel, 4);
     }
 #undef HY_GEMM
+    if (with_tail) tail->done = true;
     TL_CHECK_LAUNCH("hybrid linear");
     return TL_OK;
 }
@@ -469,15 +485,29 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
     hipLaunchKernelGGL((embed_kernel<D>), dim3(rows), dim3(256), 0, st, m.tokens, (const S *)c.embed_dev, e->x0, e->x, W, c.vocab,
                        c.embed_scale != 0.f ? c.embed_scale : 1.f);
     TL_CHECK_LAUNCH("hybrid embed");
+    bool h_ready = false;  // e->h already holds this run's first norm (it left with the product that completed the previous residual sum)
+    // the Dynamic Tanh norm that follows a residual sum: element-wise, so it can ride the completing product's epilogue
+    auto tail_for = [&](const float *w, const float *b, float alpha) {
+        NormTail t;
+        if (w && b) t.w = w, t.b = b, t.alpha = alpha, t.out = e->h;
+        return t;
+    };
     for (size_t ri = 0; ri < e->runs.size(); ++ri) {
         const Run &run = e->runs[ri];
         const tl_hybrid_layer &L = e->layers[run.layer];
+        // the first norm of the run after this one, if it is a Dynamic Tanh that reads the stream as this run leaves it
+        NormTail next_first;
+        if (!c.parallel_block && ri + 1 < e->runs.size() && !e->runs[ri + 1].enters_pass) {
+            const tl_hybrid_layer &Nx = e->layers[e->runs[ri + 1].layer];
+            if (Nx.norm_kind == TL_NORM_DYT) next_first = tail_for(Nx.norm_dev, Nx.norm_bias_dev, Nx.norm_alpha);
+        }
         if (run.enters_pass) {  // x <- W_in [x ; x0] + step[pass]
             hipLaunchKernelGGL((pack2_kernel<D>), dim3(rows), dim3(256), 0, st, e->x, e->x0, (S *)e->cat2, W);
             TL_CHECK_LAUNCH("hybrid pack2");
             HY_TRY(linear_t<D>(e->cat2, 2 * W, c.loop_in_dev, e->x, W, rows, W, 2 * W, 2, 1.f, c.loop_step_dev + (size_t)run.pass * W, 0, st));
         }
-        HY_TRY(norm_t<D>(e, L.norm_kind, L.norm_dev, L.norm_bias_dev, L.norm_alpha, L.norm_offset, e->h, nullptr, rows));
+        if (!h_ready) HY_TRY(norm_t<D>(e, L.norm_kind, L.norm_dev, L.norm_bias_dev, L.norm_alpha, L.norm_offset, e->h, nullptr, rows));
+        h_ready = false;
         const int nmix = mixer_cols(L), HV = L.heads * L.vdim;
         if (c.parallel_block) {
             const int nin = nmix + L.ff, ldcat = HV + L.ff;  // dense rows: a layer's buffers are as wide as the layer needs
@@ -490,20 +520,23 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
             // x += m ls1 * W_o mixer(norm1 x);  x += m ls2 * ff(norm2 x)
             HY_TRY(linear_t<D>(e->h, W, L.w_in_dev, e->proj, nmix, rows, nmix, W, 0, 1.f, nullptr, 0, st));
             HY_TRY(mixer_t<D>(e, ri, m, sh, nmix, HV));
-            HY_TRY(linear_t<D>(e->cat, HV, L.w_out_dev, e->x, W, rows, W, HV, L.ls1_dev ? 3 : 1, c.residual_mult, L.ls1_dev, 0, st));
+            NormTail second = (L.ff > 0 && L.norm_kind == TL_NORM_DYT) ? tail_for(L.norm2_dev, L.norm2_bias_dev, L.norm2_alpha) : NormTail{};
+            NormTail *after_mixer = L.ff > 0 ? &second : &next_first;
+            HY_TRY(linear_t<D>(e->cat, HV, L.w_out_dev, e->x, W, rows, W, HV, L.ls1_dev ? 3 : 1, c.residual_mult, L.ls1_dev, 0, st, 1, 0, 0, 0, after_mixer));
             if (L.ff > 0) {
-                HY_TRY(norm_t<D>(e, L.norm_kind, L.norm2_dev, L.norm2_bias_dev, L.norm2_alpha, L.norm_offset, e->h, nullptr, rows));
+                if (!second.done) HY_TRY(norm_t<D>(e, L.norm_kind, L.norm2_dev, L.norm2_bias_dev, L.norm2_alpha, L.norm_offset, e->h, nullptr, rows));
                 const int nin2 = ff_in_cols(L);
                 HY_TRY(linear_t<D>(e->h, W, L.w_in2_dev, e->proj, nin2, rows, nin2, W, 0, 1.f, nullptr, 0, st));
                 HY_TRY(ff_act_t<D>(e, L, rows, nin2, 0, L.ff, 0));
-                HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->x, W, rows, W, L.ff, L.ls2_dev ? 3 : 1, c.residual_mult, L.ls2_dev, 0, st));
-                if (L.ff_kind == TL_FF_MOE && L.identity > 0) {
+                if (L.ff_kind == TL_FF_MOE && L.identity > 0) {  // (before the experts' product: that one completes the sum and may carry the next norm, which overwrites h)
                     const size_t n = (size_t)rows * W;
                     hipLaunchKernelGGL((identity_axpy_kernel<D>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, e->x, (const S *)e->h, e->idw, L.ls2_dev,
                                        c.residual_mult, W, rows);
                     TL_CHECK_LAUNCH("hybrid identity experts");
                 }
+                HY_TRY(linear_t<D>(e->cat, L.ff, L.w_out2_dev, e->x, W, rows, W, L.ff, L.ls2_dev ? 3 : 1, c.residual_mult, L.ls2_dev, 0, st, 1, 0, 0, 0, &next_first));
             }
+            h_ready = next_first.done;
         }
         if (e->trace && e->trace_buf && rows <= c.max_rows)
             HY_HIP(hipMemcpyAsync(e->trace_buf + ri * (size_t)c.max_rows * W, e->x, (size_t)rows * W * 4, hipMemcpyDeviceToDevice, st));

@@ -73,11 +73,13 @@ __global__ void pack2_kernel(const float *x, const float *x0, typename D::storag
 // 64 x 64 output tile per 256-thread workgroup, 4 waves of 32 x 32 (2 x 2 MFMA 16x16 tiles), K in steps of 32 through LDS.
 // bf16: v_mfma_f32_16x16x32_bf16; fp32: v_mfma_f32_16x16x4_f32 (full fp32 products).  Any M, N, K: edges are zero-filled in LDS.
 // EPI 0: out = acc   1: out += alpha * acc   2: out = acc + bias[n]   3: out += alpha * bias[n] * acc (a per-column scale on the way into the sum)
+//     4: as 3, and the Dynamic Tanh norm of the new sum leaves with it: nout[m, n] = tanh(nalpha * out) * nw[n] + nb[n] (D rows of N; the norm is
+//        element-wise, so the product that completes a residual sum can hand the next product its input)
 // blockIdx.y = a batch of independent products of one shape (the heads of a per-head projection): operands advance by sa / sw / sc elements.
 template <typename D, int EPI>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
                                                         int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok, long sa, long sw,
-                                                        long sc) {
+                                                        long sc, const float *nw, const float *nb, float nalpha, typename D::storage *nout) {
     using S = typename D::storage;
     A += (size_t)blockIdx.y * sa, W += (size_t)blockIdx.y * sw, out += (size_t)blockIdx.y * sc;
     constexpr bool BF = sizeof(S) == 2;
@@ -177,7 +179,12 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storag
                     if constexpr (EPI == 0) *o = v;
                     else if constexpr (EPI == 1) *o += alpha * v;
                     else if constexpr (EPI == 2) *o = v + bias[gn];
-                    else *o += alpha * bias[gn] * v;
+                    else if constexpr (EPI == 3) *o += alpha * bias[gn] * v;
+                    else {
+                        const float xn = *o + alpha * bias[gn] * v;
+                        *o = xn;
+                        nout[(size_t)gm * N + gn] = D::from_float(tanhf(nalpha * xn) * nw[gn] + nb[gn]);
+                    }
                 }
             }
 }
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const typename D::storag
 template <typename D, int EPI>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const typename D::storage *A, int lda, const typename D::storage *W, float *out,
                                                         int ldc, int M, int N, int K, float alpha, const float *bias, int vec_ok, long sa, long sw,
-                                                        long sc) {
+                                                        long sc, const float *nw, const float *nb, float nalpha, typename D::storage *nout) {
     using S = typename D::storage;
     A += (size_t)blockIdx.y * sa, W += (size_t)blockIdx.y * sw, out += (size_t)blockIdx.y * sc;
     const int lane = threadIdx.x & 63;
@@ -243,7 +250,12 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const typename D::storag
                 if constexpr (EPI == 0) *o = v;
                 else if constexpr (EPI == 1) *o += alpha * v;
                 else if constexpr (EPI == 2) *o = v + bias[n];
-                else *o += alpha * bias[n] * v;
+                else if constexpr (EPI == 3) *o += alpha * bias[n] * v;
+                else {
+                    const float xn = *o + alpha * bias[n] * v;
+                    *o = xn;
+                    nout[(size_t)m * N + n] = D::from_float(tanhf(nalpha * xn) * nw[n] + nb[n]);
+                }
             }
         }
     }
