@@ -1,6 +1,6 @@
 """Plain float64 numpy restatement of the layer-list mechanisms, one function per mechanism, token by token where the
-mechanism is a recurrence.  Shares nothing with the product: it works on a dict of named arrays and a plain config dict of the
-Fonapel checkpoint format, and always processes a whole sequence from position 0.  Test infrastructure only.
+mechanism is a recurrence.  Shares nothing with the product: it works on a dict of named arrays and a plain config dict of a
+family's checkpoint format (Fonapel first, Zefapel below), and always processes a whole sequence from position 0.  Test infrastructure only.
 """
 
 from __future__ import annotations

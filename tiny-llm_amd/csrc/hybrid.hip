@@ -547,7 +547,6 @@ static int forward_t(tl_hybrid *e, const Meta &m, const StepShape &sh) {
 // final norm on the wanted rows, head product, argmax (and the slots' next input tokens)
 template <typename D>
 static int head_t(tl_hybrid *e, const Meta &m, int n_want, bool set_pending) {
-    using S = typename D::storage;
     const tl_hybrid_config &c = e->cfg;
     if (n_want <= 0) return TL_OK;
     HY_TRY(norm_t<D>(e, c.final_norm_kind, c.final_norm_dev, c.final_norm_bias_dev, c.final_norm_alpha, c.final_norm_offset, e->hsel, m.want_rows, n_want));
