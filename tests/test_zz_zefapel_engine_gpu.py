@@ -25,6 +25,9 @@ LAYERS = {
     "mlstm_dense": O.mlstm_layer(mlp=O.dense_ff()),
     "mlstm_one_head_wide_key": O.mlstm_layer(heads=1, dim=136, vdim=20),            # a wave per state column
     "mlstm_many_columns": O.mlstm_layer(heads=20, dim=72, vdim=127),                  # 16 lanes per column; the normaliser's column starts a block
+    "mlstm_32_lanes_per_column": O.mlstm_layer(heads=12, dim=40, vdim=100),               # 1,212 columns: between one wave and a DPP row per column
+    "gla_32_lanes_per_column": O.gla_layer(heads=10, dim=72, vdim=128, a_rank=8),
+    "gla_wide_key_many_columns": O.gla_layer(heads=10, dim=264, vdim=250, a_rank=8),      # 16 rows a lane at most: 32 lanes although the columns are many
     "gla": O.gla_layer(),
     "gla_moe": O.gla_layer(mlp=O.moe_ff()),
     "gla_narrow": O.gla_layer(heads=5, dim=10, vdim=7, tau=1.0, a_rank=3),
