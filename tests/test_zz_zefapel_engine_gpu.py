@@ -37,6 +37,8 @@ LAYERS = {
     "latent_frequency_ramp": O.latent_layer(rot_dim=16, scaling=(8.0, 32, 4.0, 0.5)),
     "latent_many_heads": O.latent_layer(heads=24, dim=8, vdim=8, rot_dim=4, q_rank=16, kv_rank=24),   # two blocks of 16 query heads on the one K/V head
     "latent_three_heads_odd_sizes": O.latent_layer(heads=3, dim=20, vdim=12, rot_dim=6, q_rank=9, kv_rank=26),
+    "latent_mid_tile": O.latent_layer(heads=4, dim=24, vdim=16, rot_dim=16, q_rank=24, kv_rank=104),       # key rows of 120, values of 104: the 128 / 128 tile
+    "latent_widest_tile": O.latent_layer(heads=2, dim=16, vdim=16, rot_dim=8, q_rank=16, kv_rank=216),    # key rows of 224, values of 216: the 256 / 256 tile
     "latent_wide_latent": O.latent_layer(heads=2, dim=16, vdim=16, rot_dim=8, q_rank=16, kv_rank=264),  # beyond the tile kernel: a wave per row
     "latent_moe": O.latent_layer(mlp=O.moe_ff(experts=9, identity=6, top=5, groups=5, keep=3)),
 }
